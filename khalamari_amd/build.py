@@ -1,0 +1,58 @@
+"""Builds the gfx950 shared library `libkhm_gqa_sdpa.so` in-tree with hipcc.
+
+Run as `python -m khalamari_amd.build` (or through `__graft_entry__.build()`).  hipcc cross-compiles
+for gfx950 without a GPU present; the built library is loaded by `khalamari_amd._lib`.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+PACKAGE_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC_DIR = os.path.join(PACKAGE_DIR, "csrc")
+LIB_DIR = os.path.join(PACKAGE_DIR, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libkhm_gqa_sdpa.so")
+
+SOURCES = [
+    "common.cpp",
+    "fp8_codec.cpp",
+    "sdpa_registry.cpp",
+    "replay_bucket_policy.cpp",
+    "selector.cpp",
+    "batch_metadata.cpp",
+    "components.hip",
+]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-shared",
+    "-Wall",
+    "-Wno-unused-function",
+    # packed-FP32 VALU forms are kept off for every device function in this library
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def build(verbose: bool = False, extra_flags=()) -> str:
+    os.makedirs(LIB_DIR, exist_ok=True)
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    sources = [os.path.join(CSRC_DIR, name) for name in SOURCES if os.path.exists(os.path.join(CSRC_DIR, name))]
+    command = [hipcc, *HIPCC_FLAGS, *extra_flags, "-x", "hip", *sources, "-o", LIB_PATH]
+    if verbose:
+        print(" ".join(command), flush=True)
+    result = subprocess.run(command, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    stderr = "\n".join(line for line in result.stderr.splitlines() if noise not in line)
+    if result.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({result.returncode}):\n{stderr}")
+    if verbose and stderr.strip():
+        print(stderr, file=sys.stderr)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

@@ -1,0 +1,502 @@
+// Host side of the sliced-KV and sliced-Q SDPA components and the sigmoid gate: validation, kernel
+// selection and launches.  Mirrors sliced_kv::{Config, Shape, Compute, MapInvocation, ReduceInvocation}
+// (crates/inference-backend-metal/src/components/gqa/sdpa/sliced_kv.rs:91-388,548-663),
+// sliced_q::{Config, Shape, Compute, ...} (.../sdpa/sliced_q.rs) and activation_gate::Compute
+// (.../gqa/activation_gate.rs:35-168).  Nothing here allocates or synchronizes.
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "device_params.h"
+#include "reduce_gate.hip.h"
+#include "split_kv_map.hip.h"
+
+namespace khm {
+
+constexpr int kMapWaves = 4;
+
+typedef void (*MapKernel)(const MapParams);
+typedef void (*ReduceKernel)(const ReduceParams);
+
+static MapKernel select_small_tile_kernel(uint32_t head_dim, uint32_t column_tiles) {
+    if (head_dim == 128) {
+        switch (column_tiles) {
+            case 1: return split_kv_map_kernel<128, 1, kMapWaves>;
+            case 2: return split_kv_map_kernel<128, 2, kMapWaves>;
+            case 3: return split_kv_map_kernel<128, 3, kMapWaves>;
+            case 4: return split_kv_map_kernel<128, 4, kMapWaves>;
+        }
+    } else if (head_dim == 256) {
+        switch (column_tiles) {
+            case 1: return split_kv_map_kernel<256, 1, kMapWaves>;
+            case 2: return split_kv_map_kernel<256, 2, kMapWaves>;
+            case 3: return split_kv_map_kernel<256, 3, kMapWaves>;
+            case 4: return split_kv_map_kernel<256, 4, kMapWaves>;
+        }
+    }
+    return nullptr;
+}
+
+static ReduceKernel select_reduce_kernel(uint32_t head_dim, bool ranged) {
+    if (head_dim == 128) return ranged ? split_kv_reduce_kernel<128, true> : split_kv_reduce_kernel<128, false>;
+    if (head_dim == 256) return ranged ? split_kv_reduce_kernel<256, true> : split_kv_reduce_kernel<256, false>;
+    return nullptr;
+}
+
+static DeviceReplayU32 to_device(khm_replay_u32 value) { return DeviceReplayU32{value.is_parameter, value.value}; }
+
+// ReplayU32::validate_range for Fixed values; Parameters are range-checked by whoever fills the block
+// (the reference validates them at submit: metal/stream/parameter.rs:186-204).
+static int validate_replay(khm_replay_u32 value, uint32_t min_value, uint32_t max_value, const uint32_t* block, const char* name) {
+    if (value.is_parameter) {
+        KHM_REQUIRE(block != nullptr, "%s is a replay parameter but no parameter block was given", name);
+        return KHM_OK;
+    }
+    KHM_REQUIRE(value.value >= min_value && value.value <= max_value, "%s=%u is outside its replay domain [%u, %u]", name,
+                value.value, min_value, max_value);
+    return KHM_OK;
+}
+
+static int validate_layout(const khm_page_table_layout& layout) {
+    KHM_REQUIRE(layout.num_req_slots > 0, "GQA page table requires request slots");
+    KHM_REQUIRE(layout.num_blocks > 0, "GQA page table requires blocks");
+    KHM_REQUIRE(layout.num_gqa_layers > 0, "GQA page table requires layers");
+    KHM_REQUIRE(layout.num_page_ids_per_block > 0, "GQA page table requires page ids per block");
+    return KHM_OK;
+}
+
+static uint32_t tokens_per_page_of(const khm_gqa_sdpa_config& config) {
+    const uint64_t bytes_per_token = (uint64_t)config.num_kv_heads * config.head_dim * 2 * kv_element_bytes(config.kv_dtype);
+    if (bytes_per_token == 0 || bytes_per_token > 0xffffffffull || config.page_bytes % bytes_per_token != 0) return 0;
+    return (uint32_t)(config.page_bytes / bytes_per_token);
+}
+
+// sliced_kv::Config::validate (sliced_kv.rs:101-111) / sliced_q::Config::validate (sliced_q.rs:181-196).
+static int validate_component_config(const khm_gqa_sdpa_config* config, bool sliced_q) {
+    KHM_REQUIRE(config != nullptr, "GQA SDPA config must not be null");
+    KHM_REQUIRE(config->num_q_heads > 0, "GQA SDPA requires Q heads");
+    KHM_REQUIRE(config->num_kv_heads > 0, "GQA SDPA requires KV heads");
+    KHM_REQUIRE(config->head_dim > 0, "GQA SDPA requires a head dimension");
+    KHM_REQUIRE(config->scale > 0.0f, "GQA SDPA scale must be positive");
+    KHM_REQUIRE(config->num_q_heads % config->num_kv_heads == 0, "GQA Q heads must be a multiple of KV heads");
+    KHM_REQUIRE(config->kv_dtype == KHM_DTYPE_BF16 || config->kv_dtype == KHM_DTYPE_FP8_E4M3FN,
+                "GQA K/V pages must be BF16 or FP8 E4M3FN");
+    KHM_REQUIRE(config->partial_dtype == KHM_DTYPE_BF16 || config->partial_dtype == KHM_DTYPE_F32,
+                "GQA partial outputs must be BF16 or F32");
+    const uint32_t tpp = tokens_per_page_of(*config);
+    KHM_REQUIRE(tpp > 0, "GQA page_bytes must be divisible by the K/V bytes per token");
+    if (int status = validate_layout(config->page_table_layout)) return status;
+    if (sliced_q) {
+        const bool profile = (config->head_dim == 128 && (tpp == 8 || tpp == 16)) ||
+                             (config->head_dim == 256 && (tpp == 8 || tpp == 16 || tpp == 32));
+        KHM_REQUIRE(profile,
+                    "GQA SplitKV SlicedQ supports only (head_dim, tokens_per_page) profiles (128, 8), (128, 16), (256, 8), "
+                    "(256, 16), and (256, 32), got (%u, %u)",
+                    config->head_dim, tpp);
+        KHM_REQUIRE(config->dtype == KHM_DTYPE_BF16, "GQA SplitKV SlicedQ specializes bf16");
+    } else {
+        KHM_REQUIRE(config->dtype == KHM_DTYPE_F32 || config->dtype == KHM_DTYPE_BF16, "GQA SDPA dtype must be Float32 or Bfloat16");
+    }
+    return KHM_OK;
+}
+
+static khm_sdpa_config static_config(const khm_gqa_sdpa_config& config) {
+    return khm_sdpa_config{config.dtype, config.num_q_heads, config.num_kv_heads, config.head_dim, tokens_per_page_of(config)};
+}
+
+static bool mul_overflows_u32(uint64_t a, uint64_t b, uint64_t c = 1) {
+    const __uint128_t product = (__uint128_t)a * b * c;
+    return product > 0xffffffffull;
+}
+
+struct ComputeBase {
+    khm_gqa_sdpa_config config;
+    khm_sdpa_variant variant;
+    khm_gqa_sdpa_shape shape;
+    MapKernel map;
+    ReduceKernel reduce;
+    uint32_t tokens_per_page;
+    uint32_t num_q_head_ranges;
+    bool direct;
+};
+
+static void fill_map_geometry(const ComputeBase& c, MapParams* p) {
+    const khm_gqa_sdpa_config& config = c.config;
+    p->page_bytes = config.page_bytes;
+    p->num_q_heads = config.num_q_heads;
+    p->num_kv_heads = config.num_kv_heads;
+    p->q_heads_per_kv_head = config.num_q_heads / config.num_kv_heads;
+    p->max_q_heads = c.variant.map_max_q_heads;
+    p->num_q_head_ranges = c.num_q_head_ranges;
+    p->max_q_tokens = c.variant.map_max_q_tokens;
+    p->tokens_per_page = c.tokens_per_page;
+    p->tokens_per_page_shift = ilog2_u64(c.tokens_per_page);
+    p->num_gqa_layers = config.page_table_layout.num_gqa_layers;
+    p->pages_per_request_layer = config.page_table_layout.num_blocks * config.page_table_layout.num_page_ids_per_block;
+    p->scale_log2e = config.scale * 1.4426950408889634f;
+}
+
+static int check_launch(const char* what) {
+    const hipError_t status = hipGetLastError();
+    if (status != hipSuccess) return fail(KHM_ERR_HIP, "%s launch failed: %s", what, hipGetErrorString(status));
+    return KHM_OK;
+}
+
+#define KHM_BUFFER_AT_LEAST(buffer, bytes, name)                                                                       \
+    KHM_REQUIRE((buffer).ptr != nullptr && (buffer).len_bytes >= (uint64_t)(bytes), "%s buffer holds %llu bytes, needs %llu", \
+                name, (unsigned long long)(buffer).len_bytes, (unsigned long long)(bytes))
+
+static uint64_t partial_item_size(const khm_gqa_sdpa_config& config) { return config.partial_dtype == KHM_DTYPE_F32 ? 4 : 2; }
+
+}  // namespace khm
+
+using namespace khm;
+
+struct khm_sliced_kv : ComputeBase {};
+struct khm_sliced_q : ComputeBase {};
+
+// ------------------------------------------------------------------------------------------ sizes
+
+extern "C" uint32_t khm_gqa_sdpa_num_tokens_per_page(const khm_gqa_sdpa_config* config) {
+    return config ? tokens_per_page_of(*config) : 0;
+}
+
+extern "C" uint64_t khm_gqa_sdpa_q_bytes(const khm_gqa_sdpa_config* config, const khm_gqa_sdpa_shape* shape) {
+    return (uint64_t)shape->num_total_tokens * config->num_q_heads * config->head_dim * dtype_item_size(config->dtype);
+}
+
+extern "C" uint64_t khm_gqa_sdpa_page_ids_bytes(const khm_gqa_sdpa_config* config) {
+    const khm_page_table_layout& l = config->page_table_layout;
+    return (uint64_t)l.num_req_slots * l.num_gqa_layers * l.num_blocks * l.num_page_ids_per_block * 4;
+}
+
+extern "C" uint64_t khm_sliced_kv_partial_output_stats_bytes(const khm_gqa_sdpa_config* config, const khm_gqa_sdpa_shape* shape) {
+    return (uint64_t)shape->num_total_sdpa_map_task_templates * config->num_q_heads * 4;
+}
+
+extern "C" uint64_t khm_sliced_kv_partial_output_bytes(const khm_gqa_sdpa_config* config, const khm_gqa_sdpa_shape* shape) {
+    return (uint64_t)shape->num_total_sdpa_map_task_templates * config->num_q_heads * config->head_dim * partial_item_size(*config);
+}
+
+extern "C" uint64_t khm_sliced_q_partial_output_bytes(const khm_gqa_sdpa_config* config, const khm_sdpa_variant* variant,
+                                                      const khm_gqa_sdpa_shape* shape) {
+    return (uint64_t)shape->num_total_sdpa_map_task_templates * config->num_q_heads * variant->map_max_q_tokens *
+           config->head_dim * partial_item_size(*config);
+}
+
+extern "C" uint64_t khm_sliced_q_partial_output_stats_bytes(const khm_gqa_sdpa_config* config, const khm_sdpa_variant* variant,
+                                                            const khm_gqa_sdpa_shape* shape) {
+    return (uint64_t)shape->num_total_sdpa_map_task_templates * config->num_q_heads * variant->map_max_q_tokens * 4;
+}
+
+// ------------------------------------------------------------------------------------------ sliced-KV
+
+extern "C" int khm_sliced_kv_create(const khm_gqa_sdpa_config* config, const khm_sdpa_variant* variant,
+                                    const khm_gqa_sdpa_shape* shape, khm_sliced_kv** out) {
+    clear_error();
+    if (int status = validate_component_config(config, false)) return status;
+    KHM_REQUIRE(variant != nullptr && shape != nullptr && out != nullptr, "variant, shape and out must not be null");
+    const khm_sdpa_config sdpa = static_config(*config);
+    KHM_REQUIRE(variant_supports(*variant, sdpa), "GQA SDPA execution variant does not support the config");
+    KHM_REQUIRE(variant->map_kind == KHM_MAP_SLICED_KV, "GQA SplitKV SlicedKv requires a SlicedKv execution variant");
+    // Shape::validate (sliced_kv.rs:221-234)
+    KHM_REQUIRE(shape->num_total_tokens > 0, "GQA SDPA shape requires tokens");
+    KHM_REQUIRE(shape->num_total_sdpa_map_task_templates > 0, "GQA SDPA shape requires Map task templates");
+    KHM_REQUIRE(!mul_overflows_u32(shape->num_total_tokens, config->num_q_heads, config->head_dim),
+                "GQA SDPA query/output exceeds the shader u32 count domain");
+    std::string why;
+    if (kernel_family(sdpa, *variant, config->kv_dtype, &why) != 1) return fail(KHM_ERR_UNSUPPORTED, "%s", why.c_str());
+    auto* compute = new khm_sliced_kv();
+    compute->config = *config;
+    compute->variant = *variant;
+    compute->shape = *shape;
+    compute->tokens_per_page = sdpa.tokens_per_page;
+    compute->num_q_head_ranges = div_ceil_u32(sdpa.num_q_heads / sdpa.num_kv_heads, variant->map_max_q_heads);
+    compute->direct = false;
+    compute->map = select_small_tile_kernel(config->head_dim, div_ceil_u32(variant->map_max_q_heads, 16));
+    compute->reduce = select_reduce_kernel(config->head_dim, false);
+    if (compute->map == nullptr || compute->reduce == nullptr) {
+        delete compute;
+        return fail(KHM_ERR_UNSUPPORTED, "no gfx950 sliced-KV kernel for head_dim %u", config->head_dim);
+    }
+    *out = compute;
+    return KHM_OK;
+}
+
+extern "C" void khm_sliced_kv_destroy(khm_sliced_kv* compute) { delete compute; }
+extern "C" const void* khm_sliced_kv_map_kernel_id(const khm_sliced_kv* compute) { return reinterpret_cast<const void*>(compute->map); }
+extern "C" const void* khm_sliced_kv_reduce_kernel_id(const khm_sliced_kv* compute) {
+    return reinterpret_cast<const void*>(compute->reduce);
+}
+
+extern "C" int khm_sliced_kv_map(const khm_sliced_kv* compute, const khm_sliced_kv_map_buffers* buffers,
+                                 khm_replay_u32 page_table_index, khm_replay_u32 num_active_tokens,
+                                 khm_replay_u32 num_active_kv_splits, const uint32_t* replay_parameters, void* stream) {
+    clear_error();
+    KHM_REQUIRE(compute != nullptr && buffers != nullptr, "compute and buffers must not be null");
+    const khm_gqa_sdpa_config& config = compute->config;
+    const khm_gqa_sdpa_shape& shape = compute->shape;
+    // MapInvocation::validate (sliced_kv.rs:594-613)
+    if (int s = validate_replay(page_table_index, 0, config.page_table_layout.num_gqa_layers - 1, replay_parameters, "page_table_index")) return s;
+    if (int s = validate_replay(num_active_tokens, 1, shape.num_total_tokens, replay_parameters, "num_active_tokens")) return s;
+    if (int s = validate_replay(num_active_kv_splits, 0, shape.num_total_sdpa_map_task_templates, replay_parameters, "num_active_kv_splits")) return s;
+    KHM_BUFFER_AT_LEAST(buffers->q, khm_gqa_sdpa_q_bytes(&config, &shape), "q");
+    KHM_BUFFER_AT_LEAST(buffers->kv_pages, config.page_bytes, "kv_pages");
+    KHM_BUFFER_AT_LEAST(buffers->req_slots, (uint64_t)shape.num_total_tokens * 4, "req_slots");
+    KHM_BUFFER_AT_LEAST(buffers->page_ids, khm_gqa_sdpa_page_ids_bytes(&config), "page_ids");
+    KHM_BUFFER_AT_LEAST(buffers->sdpa_map_task_templates, (uint64_t)shape.num_total_sdpa_map_task_templates * 12, "sdpa_map_task_templates");
+    KHM_BUFFER_AT_LEAST(buffers->partial_exp_sums, khm_sliced_kv_partial_output_stats_bytes(&config, &shape), "partial_exp_sums");
+    KHM_BUFFER_AT_LEAST(buffers->partial_max_logits, khm_sliced_kv_partial_output_stats_bytes(&config, &shape), "partial_max_logits");
+    KHM_BUFFER_AT_LEAST(buffers->partial_output, khm_sliced_kv_partial_output_bytes(&config, &shape), "partial_output");
+
+    MapParams p{};
+    p.q = static_cast<const uint16_t*>(buffers->q.ptr);
+    p.kv_pages = static_cast<const uint8_t*>(buffers->kv_pages.ptr);
+    p.req_slots = static_cast<const uint32_t*>(buffers->req_slots.ptr);
+    p.page_ids = static_cast<const uint32_t*>(buffers->page_ids.ptr);
+    p.visible_ranges = nullptr;
+    p.q_token_ranges = nullptr;
+    p.templates = static_cast<const uint32_t*>(buffers->sdpa_map_task_templates.ptr);
+    p.exp_sums = static_cast<float*>(buffers->partial_exp_sums.ptr);
+    p.max_logits = static_cast<float*>(buffers->partial_max_logits.ptr);
+    p.out = buffers->partial_output.ptr;
+    p.replay_parameters = replay_parameters;
+    p.layer_index = to_device(page_table_index);
+    p.num_active_tokens = to_device(num_active_tokens);
+    p.num_active_q_token_tiles = to_device(num_active_tokens);
+    p.num_active_kv_splits = to_device(num_active_kv_splits);
+    fill_map_geometry(*compute, &p);
+    p.output_mode = config.partial_dtype == KHM_DTYPE_F32 ? kMapPartialF32 : kMapPartialBf16;
+    const dim3 grid(shape.num_total_sdpa_map_task_templates, config.num_kv_heads * compute->num_q_head_ranges, 1);
+    hipLaunchKernelGGL(compute->map, grid, dim3(kMapWaves * 64), 0, static_cast<hipStream_t>(stream), p);
+    return check_launch("sliced-KV map");
+}
+
+static int launch_sliced_kv_reduce(const khm_sliced_kv* compute, const khm_sliced_kv_reduce_buffers* buffers, const khm_buffer* gates,
+                                   khm_replay_u32 num_active_tokens, const uint32_t* replay_parameters, void* stream) {
+    KHM_REQUIRE(compute != nullptr && buffers != nullptr, "compute and buffers must not be null");
+    const khm_gqa_sdpa_config& config = compute->config;
+    const khm_gqa_sdpa_shape& shape = compute->shape;
+    // ReduceInvocation::validate (sliced_kv.rs:651-662)
+    if (int s = validate_replay(num_active_tokens, 1, shape.num_total_tokens, replay_parameters, "num_active_tokens")) return s;
+    KHM_BUFFER_AT_LEAST(buffers->partial_exp_sums, khm_sliced_kv_partial_output_stats_bytes(&config, &shape), "partial_exp_sums");
+    KHM_BUFFER_AT_LEAST(buffers->partial_max_logits, khm_sliced_kv_partial_output_stats_bytes(&config, &shape), "partial_max_logits");
+    KHM_BUFFER_AT_LEAST(buffers->partial_output, khm_sliced_kv_partial_output_bytes(&config, &shape), "partial_output");
+    KHM_BUFFER_AT_LEAST(buffers->cu_sdpa_partial_outputs, ((uint64_t)shape.num_total_tokens + 1) * 4, "cu_sdpa_partial_outputs");
+    KHM_BUFFER_AT_LEAST(buffers->output, khm_gqa_sdpa_q_bytes(&config, &shape), "output");
+    if (gates != nullptr) KHM_BUFFER_AT_LEAST(*gates, khm_gqa_sdpa_q_bytes(&config, &shape), "gates");
+    ReduceParams p{};
+    p.exp_sums = static_cast<const float*>(buffers->partial_exp_sums.ptr);
+    p.max_logits = static_cast<const float*>(buffers->partial_max_logits.ptr);
+    p.partial = buffers->partial_output.ptr;
+    p.q_token_ranges = nullptr;
+    p.cu_partial_outputs = static_cast<const uint32_t*>(buffers->cu_sdpa_partial_outputs.ptr);
+    p.gates = gates ? static_cast<const uint16_t*>(gates->ptr) : nullptr;
+    p.output = static_cast<uint16_t*>(buffers->output.ptr);
+    p.replay_parameters = replay_parameters;
+    p.num_active = to_device(num_active_tokens);
+    p.num_q_heads = config.num_q_heads;
+    p.head_dim = config.head_dim;
+    p.max_q_tokens = 1;
+    p.partial_is_f32 = config.partial_dtype == KHM_DTYPE_F32;
+    const dim3 grid(shape.num_total_tokens, config.num_q_heads, 1);
+    hipLaunchKernelGGL(compute->reduce, grid, dim3(kReduceThreads), 0, static_cast<hipStream_t>(stream), p);
+    return check_launch("sliced-KV reduce");
+}
+
+extern "C" int khm_sliced_kv_reduce(const khm_sliced_kv* compute, const khm_sliced_kv_reduce_buffers* buffers,
+                                    khm_replay_u32 num_active_tokens, const uint32_t* replay_parameters, void* stream) {
+    clear_error();
+    return launch_sliced_kv_reduce(compute, buffers, nullptr, num_active_tokens, replay_parameters, stream);
+}
+
+extern "C" int khm_sliced_kv_reduce_gated(const khm_sliced_kv* compute, const khm_sliced_kv_reduce_buffers* buffers, khm_buffer gates,
+                                          khm_replay_u32 num_active_tokens, const uint32_t* replay_parameters, void* stream) {
+    clear_error();
+    return launch_sliced_kv_reduce(compute, buffers, &gates, num_active_tokens, replay_parameters, stream);
+}
+
+// ------------------------------------------------------------------------------------------ sliced-Q
+
+extern "C" int khm_sliced_q_create(const khm_gqa_sdpa_config* config, const khm_sdpa_variant* variant, const khm_gqa_sdpa_shape* shape,
+                                   int direct_output, khm_sliced_q** out) {
+    clear_error();
+    if (int status = validate_component_config(config, true)) return status;
+    KHM_REQUIRE(variant != nullptr && shape != nullptr && out != nullptr, "variant, shape and out must not be null");
+    const khm_sdpa_config sdpa = static_config(*config);
+    KHM_REQUIRE(variant_supports(*variant, sdpa), "GQA SDPA execution variant does not support the config");
+    KHM_REQUIRE(variant->map_kind != KHM_MAP_SLICED_KV, "GQA SplitKV SlicedQ requires a sliced-Q execution variant");
+    // Shape::validate (sliced_q.rs:255-273)
+    KHM_REQUIRE(shape->num_total_tokens > 0, "GQA SplitKV SlicedQ shape requires tokens");
+    KHM_REQUIRE(shape->num_total_q_token_tiles > 0 && shape->num_total_q_token_tiles <= shape->num_total_tokens,
+                "GQA SplitKV SlicedQ Q-token tiles must be in 1..=num_total_tokens");
+    KHM_REQUIRE(shape->num_total_sdpa_map_task_templates >= shape->num_total_q_token_tiles,
+                "GQA SplitKV SlicedQ needs at least one Map task template per Q-token tile");
+    KHM_REQUIRE(!mul_overflows_u32(shape->num_total_q_token_tiles, 2),
+                "GQA SplitKV SlicedQ Q-token-range metadata exceeds the shader u32 element-index domain");
+    KHM_REQUIRE(!mul_overflows_u32(shape->num_total_tokens, 2),
+                "GQA SplitKV SlicedQ visible K/V-token-range metadata exceeds the shader u32 element-index domain");
+    KHM_REQUIRE(!mul_overflows_u32(shape->num_total_sdpa_map_task_templates, 3),
+                "GQA SplitKV SlicedQ map TaskTemplate metadata exceeds the shader u32 element-index domain");
+    std::string why;
+    if (kernel_family(sdpa, *variant, config->kv_dtype, &why) != 1) return fail(KHM_ERR_UNSUPPORTED, "%s", why.c_str());
+    auto* compute = new khm_sliced_q();
+    compute->config = *config;
+    compute->variant = *variant;
+    compute->shape = *shape;
+    compute->tokens_per_page = sdpa.tokens_per_page;
+    compute->num_q_head_ranges = div_ceil_u32(sdpa.num_q_heads / sdpa.num_kv_heads, variant->map_max_q_heads);
+    compute->direct = direct_output != 0;
+    compute->map = select_small_tile_kernel(config->head_dim, div_ceil_u32(variant->map_max_q_tokens * variant->map_max_q_heads, 16));
+    compute->reduce = select_reduce_kernel(config->head_dim, true);
+    if (compute->map == nullptr || compute->reduce == nullptr) {
+        delete compute;
+        return fail(KHM_ERR_UNSUPPORTED, "no gfx950 sliced-Q kernel for head_dim %u", config->head_dim);
+    }
+    *out = compute;
+    return KHM_OK;
+}
+
+extern "C" void khm_sliced_q_destroy(khm_sliced_q* compute) { delete compute; }
+extern "C" const void* khm_sliced_q_map_kernel_id(const khm_sliced_q* compute) { return reinterpret_cast<const void*>(compute->map); }
+
+static int launch_sliced_q_map(const khm_sliced_q* compute, const khm_buffer& q, const khm_buffer& kv_pages, const khm_buffer& req_slots,
+                               const khm_buffer& page_ids, const khm_buffer& visible, const khm_buffer& ranges,
+                               const khm_buffer& templates, const khm_buffer* partial, const khm_buffer* sums,
+                               const khm_buffer* maxs, const khm_buffer* output, khm_replay_u32 page_table_index,
+                               khm_replay_u32 num_active_tokens, khm_replay_u32 num_active_q_token_tiles,
+                               khm_replay_u32 num_active_kv_splits, const uint32_t* replay_parameters, void* stream) {
+    const khm_gqa_sdpa_config& config = compute->config;
+    const khm_gqa_sdpa_shape& shape = compute->shape;
+    // MapInvocation::validate / DirectInvocation::validate (sliced_q.rs:519-545)
+    if (int s = validate_replay(page_table_index, 0, config.page_table_layout.num_gqa_layers - 1, replay_parameters, "page_table_index")) return s;
+    if (int s = validate_replay(num_active_tokens, 1, shape.num_total_tokens, replay_parameters, "num_active_tokens")) return s;
+    if (int s = validate_replay(num_active_q_token_tiles, 1, shape.num_total_q_token_tiles, replay_parameters, "num_active_q_token_tiles")) return s;
+    if (int s = validate_replay(num_active_kv_splits, 0, shape.num_total_sdpa_map_task_templates, replay_parameters, "num_active_kv_splits")) return s;
+    KHM_BUFFER_AT_LEAST(q, khm_gqa_sdpa_q_bytes(&config, &shape), "q");
+    KHM_BUFFER_AT_LEAST(kv_pages, config.page_bytes, "kv_pages");
+    KHM_BUFFER_AT_LEAST(req_slots, (uint64_t)shape.num_total_tokens * 4, "req_slots");
+    KHM_BUFFER_AT_LEAST(page_ids, khm_gqa_sdpa_page_ids_bytes(&config), "page_ids");
+    KHM_BUFFER_AT_LEAST(visible, (uint64_t)shape.num_total_tokens * 8, "visible_kv_token_ranges");
+    KHM_BUFFER_AT_LEAST(ranges, (uint64_t)shape.num_total_q_token_tiles * 8, "q_token_ranges");
+    KHM_BUFFER_AT_LEAST(templates, (uint64_t)shape.num_total_sdpa_map_task_templates * 12, "sdpa_map_task_templates");
+    MapParams p{};
+    if (output != nullptr) {
+        KHM_BUFFER_AT_LEAST(*output, khm_gqa_sdpa_q_bytes(&config, &shape), "output");
+        p.out = output->ptr;
+        p.output_mode = kMapDirectBf16;
+    } else {
+        KHM_BUFFER_AT_LEAST(*partial, khm_sliced_q_partial_output_bytes(&config, &compute->variant, &shape), "partial_output");
+        KHM_BUFFER_AT_LEAST(*sums, khm_sliced_q_partial_output_stats_bytes(&config, &compute->variant, &shape), "partial_exp_sums");
+        KHM_BUFFER_AT_LEAST(*maxs, khm_sliced_q_partial_output_stats_bytes(&config, &compute->variant, &shape), "partial_max_logits");
+        p.out = partial->ptr;
+        p.exp_sums = static_cast<float*>(sums->ptr);
+        p.max_logits = static_cast<float*>(maxs->ptr);
+        p.output_mode = config.partial_dtype == KHM_DTYPE_F32 ? kMapPartialF32 : kMapPartialBf16;
+    }
+    p.q = static_cast<const uint16_t*>(q.ptr);
+    p.kv_pages = static_cast<const uint8_t*>(kv_pages.ptr);
+    p.req_slots = static_cast<const uint32_t*>(req_slots.ptr);
+    p.page_ids = static_cast<const uint32_t*>(page_ids.ptr);
+    p.visible_ranges = static_cast<const uint32_t*>(visible.ptr);
+    p.q_token_ranges = static_cast<const uint32_t*>(ranges.ptr);
+    p.templates = static_cast<const uint32_t*>(templates.ptr);
+    p.replay_parameters = replay_parameters;
+    p.layer_index = to_device(page_table_index);
+    p.num_active_tokens = to_device(num_active_tokens);
+    p.num_active_q_token_tiles = to_device(num_active_q_token_tiles);
+    p.num_active_kv_splits = to_device(num_active_kv_splits);
+    fill_map_geometry(*compute, &p);
+    const dim3 grid(shape.num_total_sdpa_map_task_templates, config.num_kv_heads * compute->num_q_head_ranges, 1);
+    hipLaunchKernelGGL(compute->map, grid, dim3(kMapWaves * 64), 0, static_cast<hipStream_t>(stream), p);
+    return check_launch("sliced-Q map");
+}
+
+extern "C" int khm_sliced_q_map(const khm_sliced_q* compute, const khm_sliced_q_map_buffers* buffers, khm_replay_u32 page_table_index,
+                                khm_replay_u32 num_active_tokens, khm_replay_u32 num_active_q_token_tiles,
+                                khm_replay_u32 num_active_kv_splits, const uint32_t* replay_parameters, void* stream) {
+    clear_error();
+    KHM_REQUIRE(compute != nullptr && buffers != nullptr, "compute and buffers must not be null");
+    KHM_REQUIRE(!compute->direct, "GQA SplitKV SlicedQ direct-output compute cannot record a partial Map");
+    return launch_sliced_q_map(compute, buffers->q, buffers->kv_pages, buffers->req_slots, buffers->page_ids,
+                               buffers->visible_kv_token_ranges, buffers->q_token_ranges, buffers->sdpa_map_task_templates,
+                               &buffers->partial_output, &buffers->partial_exp_sums, &buffers->partial_max_logits, nullptr,
+                               page_table_index, num_active_tokens, num_active_q_token_tiles, num_active_kv_splits,
+                               replay_parameters, stream);
+}
+
+extern "C" int khm_sliced_q_direct(const khm_sliced_q* compute, const khm_sliced_q_direct_buffers* buffers,
+                                   khm_replay_u32 page_table_index, khm_replay_u32 num_active_tokens,
+                                   khm_replay_u32 num_active_q_token_tiles, const uint32_t* replay_parameters, void* stream) {
+    clear_error();
+    KHM_REQUIRE(compute != nullptr && buffers != nullptr, "compute and buffers must not be null");
+    KHM_REQUIRE(compute->direct, "GQA SplitKV SlicedQ direct output requires a direct-output compute");
+    // One direct Map owns each Q range: both padded domains have the same extent (sdpa.rs:564-568).
+    KHM_REQUIRE(compute->shape.num_total_sdpa_map_task_templates == compute->shape.num_total_q_token_tiles,
+                "GQA direct output requires one Map task template per Q-token tile");
+    return launch_sliced_q_map(compute, buffers->q, buffers->kv_pages, buffers->req_slots, buffers->page_ids,
+                               buffers->visible_kv_token_ranges, buffers->q_token_ranges, buffers->sdpa_map_task_templates, nullptr,
+                               nullptr, nullptr, &buffers->output, page_table_index, num_active_tokens, num_active_q_token_tiles,
+                               num_active_q_token_tiles, replay_parameters, stream);
+}
+
+extern "C" int khm_sliced_q_reduce(const khm_sliced_q* compute, const khm_sliced_q_reduce_buffers* buffers,
+                                   khm_replay_u32 num_active_q_token_tiles, const uint32_t* replay_parameters, void* stream) {
+    clear_error();
+    KHM_REQUIRE(compute != nullptr && buffers != nullptr, "compute and buffers must not be null");
+    KHM_REQUIRE(!compute->direct, "GQA SplitKV SlicedQ direct-output compute has no Reduce");
+    const khm_gqa_sdpa_config& config = compute->config;
+    const khm_gqa_sdpa_shape& shape = compute->shape;
+    // ReduceInvocation::validate (sliced_q.rs:603-618)
+    if (int s = validate_replay(num_active_q_token_tiles, 1, shape.num_total_q_token_tiles, replay_parameters, "num_active_q_token_tiles")) return s;
+    KHM_BUFFER_AT_LEAST(buffers->partial_output, khm_sliced_q_partial_output_bytes(&config, &compute->variant, &shape), "partial_output");
+    KHM_BUFFER_AT_LEAST(buffers->partial_exp_sums, khm_sliced_q_partial_output_stats_bytes(&config, &compute->variant, &shape), "partial_exp_sums");
+    KHM_BUFFER_AT_LEAST(buffers->partial_max_logits, khm_sliced_q_partial_output_stats_bytes(&config, &compute->variant, &shape), "partial_max_logits");
+    KHM_BUFFER_AT_LEAST(buffers->q_token_ranges, (uint64_t)shape.num_total_q_token_tiles * 8, "q_token_ranges");
+    KHM_BUFFER_AT_LEAST(buffers->cu_sdpa_partial_outputs, ((uint64_t)shape.num_total_q_token_tiles + 1) * 4, "cu_sdpa_partial_outputs");
+    KHM_BUFFER_AT_LEAST(buffers->output, khm_gqa_sdpa_q_bytes(&config, &shape), "output");
+    ReduceParams p{};
+    p.exp_sums = static_cast<const float*>(buffers->partial_exp_sums.ptr);
+    p.max_logits = static_cast<const float*>(buffers->partial_max_logits.ptr);
+    p.partial = buffers->partial_output.ptr;
+    p.q_token_ranges = static_cast<const uint32_t*>(buffers->q_token_ranges.ptr);
+    p.cu_partial_outputs = static_cast<const uint32_t*>(buffers->cu_sdpa_partial_outputs.ptr);
+    p.gates = nullptr;
+    p.output = static_cast<uint16_t*>(buffers->output.ptr);
+    p.replay_parameters = replay_parameters;
+    p.num_active = to_device(num_active_q_token_tiles);
+    p.num_q_heads = config.num_q_heads;
+    p.head_dim = config.head_dim;
+    p.max_q_tokens = compute->variant.map_max_q_tokens;
+    p.partial_is_f32 = config.partial_dtype == KHM_DTYPE_F32;
+    const dim3 grid(shape.num_total_q_token_tiles, config.num_q_heads, 1);
+    hipLaunchKernelGGL(compute->reduce, grid, dim3(kReduceThreads), 0, static_cast<hipStream_t>(stream), p);
+    return check_launch("sliced-Q reduce");
+}
+
+// ------------------------------------------------------------------------------------------ gate
+
+extern "C" int khm_gqa_activation_gate(uint32_t dtype, uint32_t num_q_heads, uint32_t head_dim, uint32_t num_total_tokens,
+                                       khm_buffer attention_output, khm_buffer gates, khm_buffer output,
+                                       khm_replay_u32 num_active_tokens, const uint32_t* replay_parameters, void* stream) {
+    clear_error();
+    KHM_REQUIRE(dtype == KHM_DTYPE_F32 || dtype == KHM_DTYPE_BF16, "unsupported GQA activation gate dtype");
+    KHM_REQUIRE(num_q_heads > 0 && head_dim > 0 && num_total_tokens > 0, "GQA activation/gate requires tokens, heads and a head dimension");
+    KHM_REQUIRE(!mul_overflows_u32(num_total_tokens, num_q_heads, head_dim), "GQA activation/gate exceeds the shader u32 count domain");
+    if (int s = validate_replay(num_active_tokens, 1, num_total_tokens, replay_parameters, "num_active_tokens")) return s;
+    const uint64_t values = (uint64_t)num_total_tokens * num_q_heads * head_dim;
+    const uint64_t bytes = values * dtype_item_size(dtype);
+    KHM_BUFFER_AT_LEAST(attention_output, bytes, "attention_output");
+    KHM_BUFFER_AT_LEAST(gates, bytes, "gates");
+    KHM_BUFFER_AT_LEAST(output, bytes, "output");
+    GateParams p{};
+    p.attention = attention_output.ptr;
+    p.gates = gates.ptr;
+    p.output = output.ptr;
+    p.replay_parameters = replay_parameters;
+    p.num_active_tokens = to_device(num_active_tokens);
+    p.values_per_token = num_q_heads * head_dim;
+    p.is_f32 = dtype == KHM_DTYPE_F32;
+    const uint32_t blocks = (uint32_t)((values + 255) / 256);
+    hipLaunchKernelGGL(activation_gate_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    return check_launch("activation gate");
+}

@@ -1,0 +1,479 @@
+// Split-KV Map kernel for decode and speculative-verify blocks on gfx950 (wave64, bf16 MFMA).
+//
+// Replaces gqa_sdpa_sliced_kv_map (crates/inference-backend-metal/src/components/metal/
+// gqa_sdpa_sliced_kv_map.metal:36-211) and, for small Q tiles, gqa_sdpa_sliced_q_map
+// (.../gqa_sdpa_sliced_q_map.metal:29-284).  Same task ABI: one block per
+// (map task template, KV head, Q-head range); same partial-state contract: normalized partial,
+// exp-sum, natural-log max, canonical empty state (0, -inf, 0), inactive coordinates untouched.
+//
+// Work shape.  The block's Q coordinates (q_token, q_head) are the N columns of 16-wide MFMA
+// tiles (NT tiles).  KV is walked in 16-token tiles; wave w of the block takes tiles
+// w, w + NWAVES, ...  Per tile a wave computes
+//     S^T[token][col] = K[token][:] . Q[col][:]           v_mfma_f32_16x16x32_bf16, K as the A operand
+//     online softmax per column (exp2 domain, f32)
+//     O^T[dim][col]  += V^T[dim][token] . P^T[token][col]  v_mfma_f32_16x16x16_bf16
+// Computing S transposed makes the softmax weights land in exactly the register layout the
+// second MFMA wants for its B operand, so P never moves between lanes, and the per-column
+// rescale factor is a per-lane scalar.
+//
+// Memory.  K rows go from HBM straight into the A-operand layout (each lane: one token row,
+// 16 B per k-step).  V rows are loaded as fully coalesced 16-byte chunks, written to a
+// wave-private LDS tile and read back transposed (4 tokens of one dim per lane).  Loads for
+// tile j+2 are issued before tile j is consumed (three register buffers).  Page ids are read
+// once per 64 tiles into a register and broadcast with v_readlane, so the page-table lookup is
+// never on the critical path of a K/V load.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "device_params.h"
+
+namespace khm {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t resolve_u32(DeviceReplayU32 r, const uint32_t* params) {
+    return r.is_parameter ? params[r.value] : r.value;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits) { return __uint_as_float(bits << 16); }
+
+// Round-to-nearest-even f32 -> bf16 bits (v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float v) { return (uint16_t)(pack_bf16x2(v, 0.0f) & 0xffffu); }
+
+template <int D>
+struct KvTile {
+    uint4 k[D / 32];  // A-operand fragments: token row (lane & 15), dims ks*32 + (lane >> 4)*8 .. +8
+    uint4 v[D / 32];  // coalesced chunks: row i*(512/D) + lane/(D/8), dims (lane % (D/8))*8 .. +8
+    uint32_t first_token;
+};
+
+template <int D, int NT, int NWAVES>
+struct MapSmem {
+    static constexpr int kVRowBytes = D * 2 + 8;           // +8 B: conflict-free transposed reads
+    static constexpr int kVBytes = NWAVES * 16 * kVRowBytes;
+    static constexpr int kCols = NT * 16;
+    static constexpr int kORowFloats = D + 4;
+    static constexpr int kOBytes = kCols * kORowFloats * 4;
+    static constexpr int kUnionBytes = kVBytes > kOBytes ? kVBytes : kOBytes;
+    static constexpr int kQRowBytes = D * 2 + 16;
+    static constexpr int kQBytes = kCols * kQRowBytes;
+    static constexpr int kStatsBytes = (NWAVES + 1) * kCols * 2 * 4;
+    static constexpr int kTotal = kUnionBytes + kQBytes + kStatsBytes;
+};
+
+template <int D, int NT, int NWAVES>
+__global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapParams p) {
+    constexpr int KS = D / 32;
+    constexpr int MT = D / 16;
+    constexpr int COLS = NT * 16;
+    constexpr int LANES_PER_ROW = D / 8;          // 16-byte chunks per K/V row
+    constexpr int ROWS_PER_LOAD = 64 / LANES_PER_ROW;
+    using Smem = MapSmem<D, NT, NWAVES>;
+    constexpr bool kQInRegs = (NT == 1);
+
+    __shared__ __align__(16) unsigned char smem[Smem::kTotal];
+    unsigned char* v_lds_all = smem;
+    float* o_lds = reinterpret_cast<float*>(smem);
+    unsigned char* q_lds = smem + Smem::kUnionBytes;
+    float* stats_lds = reinterpret_cast<float*>(smem + Smem::kUnionBytes + Smem::kQBytes);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15;
+    const int g = lane >> 4;
+
+    // ---- task decode (uniform) -------------------------------------------------------------
+    const uint32_t task = blockIdx.x;
+    if (task >= resolve_u32(p.num_active_kv_splits, p.replay_parameters)) return;
+    const uint32_t range_index = p.templates[3 * (uint64_t)task];
+    if (range_index >= resolve_u32(p.num_active_q_token_tiles, p.replay_parameters)) return;
+    uint32_t flat_begin, flat_end;
+    if (p.q_token_ranges != nullptr) {
+        flat_begin = p.q_token_ranges[2 * (uint64_t)range_index];
+        flat_end = p.q_token_ranges[2 * (uint64_t)range_index + 1];
+    } else {
+        flat_begin = range_index;
+        flat_end = range_index + 1;
+    }
+    const uint32_t num_active_tokens = resolve_u32(p.num_active_tokens, p.replay_parameters);
+    if (flat_begin >= num_active_tokens || flat_end > num_active_tokens || flat_end <= flat_begin) return;
+    uint32_t num_q = flat_end - flat_begin;
+    if (num_q > p.max_q_tokens) num_q = p.max_q_tokens;
+    const uint32_t kv_begin = p.templates[3 * (uint64_t)task + 1];
+    const uint32_t kv_end = p.templates[3 * (uint64_t)task + 2];
+    const uint32_t req_slot = p.req_slots[flat_begin];
+    const uint32_t layer = resolve_u32(p.layer_index, p.replay_parameters);
+
+    const uint32_t head_range = blockIdx.y % p.num_q_head_ranges;
+    const uint32_t kv_head = blockIdx.y / p.num_q_head_ranges;
+    const uint32_t head_range_begin = head_range * p.max_q_heads;
+    const uint32_t heads_left = p.q_heads_per_kv_head - head_range_begin;
+    const uint32_t num_heads = heads_left < p.max_q_heads ? heads_left : p.max_q_heads;
+    const uint32_t first_q_head = kv_head * p.q_heads_per_kv_head + head_range_begin;
+
+    // ---- per-lane column facts -------------------------------------------------------------
+    // Column c = token_offset * max_q_heads + local_head.
+    uint32_t col_lo[NT], col_hi[NT];
+    bool col_active[NT];
+    uint32_t blk_lo = 0xffffffffu, blk_hi = 0u, all_lo = 0u, all_hi = 0xffffffffu;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const uint32_t c = nt * 16 + r16;
+        const uint32_t token_offset = c / p.max_q_heads;
+        const uint32_t local_head = c - token_offset * p.max_q_heads;
+        col_active[nt] = token_offset < num_q && local_head < num_heads;
+        uint32_t lo = kv_begin, hi = kv_end;
+        if (col_active[nt] && p.visible_ranges != nullptr) {
+            const uint64_t token = flat_begin + token_offset;
+            const uint32_t vis_lo = p.visible_ranges[2 * token];
+            const uint32_t vis_hi = p.visible_ranges[2 * token + 1];
+            lo = vis_lo > lo ? vis_lo : lo;
+            hi = vis_hi < hi ? vis_hi : hi;
+        }
+        if (hi < lo) hi = lo;
+        col_lo[nt] = lo;
+        col_hi[nt] = hi;
+        if (col_active[nt]) {
+            if (hi > lo) {
+                blk_lo = lo < blk_lo ? lo : blk_lo;
+                blk_hi = hi > blk_hi ? hi : blk_hi;
+            }
+            all_lo = lo > all_lo ? lo : all_lo;
+            all_hi = hi < all_hi ? hi : all_hi;
+        }
+    }
+#pragma unroll
+    for (int offset = 1; offset < 16; offset <<= 1) {
+        uint32_t other;
+        other = __shfl_xor(blk_lo, offset); blk_lo = other < blk_lo ? other : blk_lo;
+        other = __shfl_xor(blk_hi, offset); blk_hi = other > blk_hi ? other : blk_hi;
+        other = __shfl_xor(all_lo, offset); all_lo = other > all_lo ? other : all_lo;
+        other = __shfl_xor(all_hi, offset); all_hi = other < all_hi ? other : all_hi;
+    }
+    blk_lo = __builtin_amdgcn_readfirstlane(blk_lo);
+    blk_hi = __builtin_amdgcn_readfirstlane(blk_hi);
+    all_lo = __builtin_amdgcn_readfirstlane(all_lo);
+    all_hi = __builtin_amdgcn_readfirstlane(all_hi);
+    {
+        // Never walk past the request's page table.
+        const uint64_t table_tokens = (uint64_t)p.pages_per_request_layer << p.tokens_per_page_shift;
+        if (blk_hi > table_tokens) blk_hi = (uint32_t)table_tokens;
+    }
+
+    // ---- Q fragments -----------------------------------------------------------------------
+    // B operand of S^T = K.Q^T: lane holds Q[col = lane & 15][dims ks*32 + g*8 .. +8].
+    uint4 q_frag[kQInRegs ? KS : 1];
+    if constexpr (kQInRegs) {
+        const uint32_t c = r16;
+        const uint32_t token_offset = c / p.max_q_heads;
+        const uint32_t local_head = c - token_offset * p.max_q_heads;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) q_frag[ks] = make_uint4(0, 0, 0, 0);
+        if (col_active[0]) {
+            const uint16_t* row = p.q + ((uint64_t)(flat_begin + token_offset) * p.num_q_heads + first_q_head + local_head) * D;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) q_frag[ks] = *reinterpret_cast<const uint4*>(row + ks * 32 + g * 8);
+        }
+    } else {
+        for (int index = tid; index < COLS * LANES_PER_ROW; index += NWAVES * 64) {
+            const uint32_t c = index / LANES_PER_ROW;
+            const uint32_t chunk = index - c * LANES_PER_ROW;
+            const uint32_t token_offset = c / p.max_q_heads;
+            const uint32_t local_head = c - token_offset * p.max_q_heads;
+            uint4 value = make_uint4(0, 0, 0, 0);
+            if (token_offset < num_q && local_head < num_heads) {
+                const uint16_t* row = p.q + ((uint64_t)(flat_begin + token_offset) * p.num_q_heads + first_q_head + local_head) * D;
+                value = *reinterpret_cast<const uint4*>(row + chunk * 8);
+            }
+            *reinterpret_cast<uint4*>(q_lds + c * Smem::kQRowBytes + chunk * 16) = value;
+        }
+        __syncthreads();
+    }
+
+    // ---- tile schedule ---------------------------------------------------------------------
+    const uint32_t tile_first = blk_lo >> 4;
+    const uint32_t num_tiles = blk_hi > blk_lo ? ((blk_hi - 1) >> 4) - tile_first + 1 : 0;
+    const uint32_t num_wave_tiles = num_tiles > (uint32_t)wave ? (num_tiles - wave + NWAVES - 1) / NWAVES : 0;
+
+    const uint32_t* table = p.page_ids + ((uint64_t)req_slot * p.num_gqa_layers + layer) * p.pages_per_request_layer;
+    const uint32_t tpp = p.tokens_per_page;
+    const uint32_t tpp_shift = p.tokens_per_page_shift;
+    const uint64_t kv_head_row0_k = ((uint64_t)kv_head * tpp) * (D * 2);
+    const uint64_t kv_head_row0_v = ((uint64_t)(p.num_kv_heads + kv_head) * tpp) * (D * 2);
+
+    // Page ids of 64 consecutive wave tiles per register; two registers alternate.
+    uint32_t ids_a[2] = {0, 0}, ids_b[2] = {0, 0};
+    auto load_ids = [&](uint32_t chunk, uint32_t (&ids)[2]) {
+        const uint32_t j = chunk * 64 + lane;
+        if (j < num_wave_tiles) {
+            const uint32_t token = (tile_first + wave + NWAVES * j) << 4;
+            const uint32_t last_page = p.pages_per_request_layer - 1;
+            const uint32_t page0 = token >> tpp_shift;
+            const uint32_t page1 = (token + 8) >> tpp_shift;
+            ids[0] = table[page0 < last_page ? page0 : last_page];
+            ids[1] = table[page1 < last_page ? page1 : last_page];
+        }
+    };
+    load_ids(0, ids_a);
+    if (num_wave_tiles > 64) load_ids(1, ids_b);
+
+    auto load_tile = [&](uint32_t j, KvTile<D>& tile) {
+        const uint32_t chunk = j >> 6;
+        if ((j & 63) == 0 && chunk >= 1 && (chunk + 1) * 64 < num_wave_tiles) {
+            if ((chunk + 1) & 1) load_ids(chunk + 1, ids_b); else load_ids(chunk + 1, ids_a);
+        }
+        const uint32_t sel0 = (chunk & 1) ? ids_b[0] : ids_a[0];
+        const uint32_t sel1 = (chunk & 1) ? ids_b[1] : ids_a[1];
+        uint32_t id0 = __builtin_amdgcn_readlane(sel0, j & 63);
+        uint32_t id1 = __builtin_amdgcn_readlane(sel1, j & 63);
+        const uint32_t first_token = (tile_first + wave + NWAVES * j) << 4;
+        if (tpp == 8) {
+            // A tile spans two 8-token pages; the half outside the block's KV range may have no
+            // page assigned (its table entry can hold anything), so it borrows the other half's page.
+            // Its K rows are masked and its V rows zeroed below.
+            if (first_token + 8 >= blk_hi) id1 = id0;
+            if (first_token + 8 <= blk_lo) id0 = id1;
+        }
+        tile.first_token = first_token;
+        {
+            const uint32_t row = r16;
+            const uint32_t in_page = (first_token + row) & (tpp - 1);
+            const uint64_t page = (row >= 8 ? id1 : id0);
+            const unsigned char* base = p.kv_pages + page * p.page_bytes + kv_head_row0_k + (uint64_t)in_page * (D * 2) + g * 16;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) tile.k[ks] = *reinterpret_cast<const uint4*>(base + ks * 64);
+        }
+        {
+            const uint32_t row_in_load = lane / LANES_PER_ROW;
+            const uint32_t chunk_in_row = lane % LANES_PER_ROW;
+#pragma unroll
+            for (int i = 0; i < KS; ++i) {
+                const uint32_t row = i * ROWS_PER_LOAD + row_in_load;
+                const uint32_t in_page = (first_token + row) & (tpp - 1);
+                const uint64_t page = (row >= 8 ? id1 : id0);
+                const unsigned char* source = p.kv_pages + page * p.page_bytes + kv_head_row0_v + (uint64_t)in_page * (D * 2) + chunk_in_row * 16;
+                tile.v[i] = *reinterpret_cast<const uint4*>(source);
+            }
+        }
+    };
+
+    // ---- online-softmax state --------------------------------------------------------------
+    f32x4 acc[NT][MT];
+    float run_max[NT], run_sum[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        run_max[nt] = -INFINITY;
+        run_sum[nt] = 0.0f;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    unsigned char* v_lds = v_lds_all + wave * 16 * Smem::kVRowBytes;
+
+    auto compute_tile = [&](const KvTile<D>& tile) {
+        const uint32_t first_token = tile.first_token;
+        // S^T = K . Q^T
+        f32x4 s[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) s[nt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const bf16x8 a = __builtin_bit_cast(bf16x8, tile.k[ks]);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                uint4 b_bits;
+                if constexpr (kQInRegs) {
+                    b_bits = q_frag[ks];
+                } else {
+                    b_bits = *reinterpret_cast<const uint4*>(q_lds + (nt * 16 + r16) * Smem::kQRowBytes + (ks * 32 + g * 8) * 2);
+                }
+                s[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, b_bits), s[nt], 0, 0, 0);
+            }
+        }
+        const bool interior = first_token >= all_lo && first_token + 16 <= all_hi;
+        uint32_t p_bits[NT][2];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = s[nt][i] * p.scale_log2e;
+            if (!interior) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t token = first_token + g * 4 + i;
+                    v[i] = (token >= col_lo[nt] && token < col_hi[nt]) ? v[i] : -INFINITY;
+                }
+            }
+            float tile_max = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
+            const float next_max = fmaxf(run_max[nt], tile_max);
+            const float safe_max = next_max == -INFINITY ? 0.0f : next_max;
+            const float alpha = fast_exp2(run_max[nt] - safe_max);
+            run_max[nt] = next_max;
+            float e[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) e[i] = fast_exp2(v[i] - safe_max);
+            run_sum[nt] = run_sum[nt] * alpha + ((e[0] + e[1]) + (e[2] + e[3]));
+            p_bits[nt][0] = pack_bf16x2(e[0], e[1]);
+            p_bits[nt][1] = pack_bf16x2(e[2], e[3]);
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[nt][mt] *= alpha;
+            }
+        }
+        // V tile -> wave-private LDS (rows outside the block's KV range are zeroed: an unused
+        // page slot may hold anything, and 0 * NaN would poison the accumulator).
+        {
+            const uint32_t row_in_load = lane / LANES_PER_ROW;
+            const uint32_t chunk_in_row = lane % LANES_PER_ROW;
+            const bool edge = first_token < blk_lo || first_token + 16 > blk_hi;
+#pragma unroll
+            for (int i = 0; i < KS; ++i) {
+                const uint32_t row = i * ROWS_PER_LOAD + row_in_load;
+                uint4 value = tile.v[i];
+                if (edge) {
+                    const uint32_t token = first_token + row;
+                    if (token < blk_lo || token >= blk_hi) value = make_uint4(0, 0, 0, 0);
+                }
+                uint2* target = reinterpret_cast<uint2*>(v_lds + row * Smem::kVRowBytes + chunk_in_row * 16);
+                target[0] = make_uint2(value.x, value.y);
+                target[1] = make_uint2(value.z, value.w);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // O^T += V^T . P^T
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const unsigned char* column = v_lds + (g * 4) * Smem::kVRowBytes + (mt * 16 + r16) * 2;
+            s16x4 a;
+            a[0] = *reinterpret_cast<const short*>(column);
+            a[1] = *reinterpret_cast<const short*>(column + Smem::kVRowBytes);
+            a[2] = *reinterpret_cast<const short*>(column + 2 * Smem::kVRowBytes);
+            a[3] = *reinterpret_cast<const short*>(column + 3 * Smem::kVRowBytes);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const uint2 b_bits = make_uint2(p_bits[nt][0], p_bits[nt][1]);
+                acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, __builtin_bit_cast(s16x4, b_bits), acc[nt][mt], 0, 0, 0);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+
+    // ---- main loop: three rotating register buffers, loads two tiles ahead -----------------
+    if (num_wave_tiles > 0) {
+        KvTile<D> t0, t1, t2;
+        load_tile(0, t0);
+        if (num_wave_tiles > 1) load_tile(1, t1);
+        uint32_t j = 0;
+        while (true) {
+            if (j + 2 < num_wave_tiles) load_tile(j + 2, t2);
+            compute_tile(t0);
+            if (++j >= num_wave_tiles) break;
+            if (j + 2 < num_wave_tiles) load_tile(j + 2, t0);
+            compute_tile(t1);
+            if (++j >= num_wave_tiles) break;
+            if (j + 2 < num_wave_tiles) load_tile(j + 2, t1);
+            compute_tile(t2);
+            if (++j >= num_wave_tiles) break;
+        }
+    }
+
+    // ---- merge the waves of the block ------------------------------------------------------
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        run_sum[nt] += __shfl_xor(run_sum[nt], 16);
+        run_sum[nt] += __shfl_xor(run_sum[nt], 32);
+        if (g == 0) {
+            stats_lds[(wave * COLS + nt * 16 + r16) * 2] = run_max[nt];
+            stats_lds[(wave * COLS + nt * 16 + r16) * 2 + 1] = run_sum[nt];
+        }
+    }
+    __syncthreads();  // also: every wave is done with its V staging tile
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int c = nt * 16 + r16;
+        float global_max = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < NWAVES; ++w) global_max = fmaxf(global_max, stats_lds[(w * COLS + c) * 2]);
+        float global_sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NWAVES; ++w) {
+            const float wave_sum = stats_lds[(w * COLS + c) * 2 + 1];
+            if (wave_sum > 0.0f) global_sum += wave_sum * fast_exp2(stats_lds[(w * COLS + c) * 2] - global_max);
+        }
+        const float own = (run_sum[nt] > 0.0f && global_sum > 0.0f) ? fast_exp2(run_max[nt] - global_max) / global_sum : 0.0f;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] *= own;
+        if (wave == 0 && g == 0) {
+            stats_lds[(NWAVES * COLS + c) * 2] = global_sum > 0.0f ? global_max * 0.6931471805599453f : -INFINITY;
+            stats_lds[(NWAVES * COLS + c) * 2 + 1] = global_sum;
+        }
+    }
+    for (int w = 0; w < NWAVES; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    float* cell = o_lds + (nt * 16 + r16) * Smem::kORowFloats + mt * 16 + g * 4;
+                    f32x4 value = acc[nt][mt];
+                    if (w > 0) value += *reinterpret_cast<const f32x4*>(cell);
+                    *reinterpret_cast<f32x4*>(cell) = value;
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- write the block's partial state or final output ------------------------------------
+    const uint32_t mode = p.output_mode;
+    for (int index = tid; index < COLS * (D / 4); index += NWAVES * 64) {
+        const uint32_t c = index / (D / 4);
+        const uint32_t d = (index - c * (D / 4)) * 4;
+        const uint32_t token_offset = c / p.max_q_heads;
+        const uint32_t local_head = c - token_offset * p.max_q_heads;
+        if (token_offset >= num_q || local_head >= num_heads) continue;
+        const f32x4 value = *reinterpret_cast<const f32x4*>(o_lds + c * Smem::kORowFloats + d);
+        const uint32_t q_head = first_q_head + local_head;
+        uint64_t state;
+        if (mode == kMapDirectBf16) {
+            state = (uint64_t)(flat_begin + token_offset) * p.num_q_heads + q_head;
+        } else {
+            state = ((uint64_t)task * p.num_q_heads + q_head) * p.max_q_tokens + token_offset;
+        }
+        if (mode == kMapPartialF32) {
+            *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.out) + state * D + d) = value;
+        } else {
+            const uint2 packed = make_uint2(pack_bf16x2(value[0], value[1]), pack_bf16x2(value[2], value[3]));
+            *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.out) + state * D + d) = packed;
+        }
+    }
+    if (mode != kMapDirectBf16 && tid < COLS) {
+        const uint32_t c = tid;
+        const uint32_t token_offset = c / p.max_q_heads;
+        const uint32_t local_head = c - token_offset * p.max_q_heads;
+        if (token_offset < num_q && local_head < num_heads) {
+            const uint64_t state = ((uint64_t)task * p.num_q_heads + first_q_head + local_head) * p.max_q_tokens + token_offset;
+            p.max_logits[state] = stats_lds[(NWAVES * COLS + c) * 2];
+            p.exp_sums[state] = stats_lds[(NWAVES * COLS + c) * 2 + 1];
+        }
+    }
+}
+
+}  // namespace khm

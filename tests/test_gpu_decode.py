@@ -1,0 +1,51 @@
+"""GPU parity of the decode (sliced-KV) path against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+from khalamari_amd._lib import DTYPE_BF16, DTYPE_F32
+
+from . import gpu_runner, helpers
+
+pytestmark = pytest.mark.gpu
+
+
+def _decode_case(device, *, hq, hkv, d, tpp, histories, kv_slice, seed, partial_dtype=DTYPE_BF16, **kw):
+    q_lens = [1] * len(histories)
+    w = helpers.make_workload(num_q_heads=hq, num_kv_heads=hkv, head_dim=d, tokens_per_page=tpp, histories=histories,
+                              q_lens=q_lens, seed=seed, **kw)
+    _, templates, cu = helpers.fixed_slice_plan(histories, q_lens, 1, kv_slice)
+    print(f"decode case hq={hq} hkv={hkv} d={d} tpp={tpp} histories={histories} slice={kv_slice} seed={seed}", flush=True)
+    actual, _ = gpu_runner.run_sliced_kv(w, templates, cu, device, partial_dtype=partial_dtype)
+    expected = helpers.expected_output(w)
+    return helpers.assert_parity(actual, expected, f"decode d={d} tpp={tpp}")
+
+
+def test_config1_single_sequence_identity_pages(device):
+    """BASELINE config 1: batch 1, Hq32/Hkv8/D128, context 1024, page 16, identity page table."""
+    stats = _decode_case(device, hq=32, hkv=8, d=128, tpp=16, histories=[1023], kv_slice=256, seed=1, permute=False)
+    print(stats)
+
+
+@pytest.mark.parametrize("partial_dtype", [DTYPE_BF16, DTYPE_F32])
+def test_ragged_batch_permuted_pages(device, partial_dtype):
+    """Config-2 shape at reduced size: ragged contexts, shared permuted pool, 512-token partitions."""
+    _decode_case(device, hq=64, hkv=8, d=128, tpp=16, histories=[511, 700, 1500, 33, 0, 15, 16, 2047], kv_slice=512,
+                 seed=2, partial_dtype=partial_dtype)
+
+
+def test_d256_ratio6(device):
+    """Config-3 geometry (Hq24/Hkv4/D256) at reduced context with 2048-token partitions."""
+    _decode_case(device, hq=24, hkv=4, d=256, tpp=16, histories=[5000, 2047, 2048, 100], kv_slice=2048, seed=3)
+
+
+@pytest.mark.parametrize("tpp", [8, 32])
+@pytest.mark.parametrize("d", [128, 256])
+def test_other_page_sizes(device, d, tpp):
+    if d == 128 and tpp == 32:
+        pytest.skip("(128, 32) is not a reference profile")
+    _decode_case(device, hq=12, hkv=2, d=d, tpp=tpp, histories=[70, 9, 300], kv_slice=64, seed=4 + tpp)
+
+
+def test_unaligned_slices_and_nan_garbage(device):
+    """Slices that do not align with pages, and NaN in every unused page slot."""
+    _decode_case(device, hq=16, hkv=2, d=128, tpp=16, histories=[130, 64, 7], kv_slice=65, seed=9, garbage_bits=0x7FC0)
