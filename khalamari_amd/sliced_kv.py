@@ -108,8 +108,8 @@ class Compute:
 
     def __del__(self):
         handle = getattr(self, "_handle", None)
-        if handle:
-            _lib.lib().khm_sliced_kv_destroy(handle)
+        if handle and _lib is not None and getattr(_lib, "_lib", None) is not None:
+            _lib._lib.khm_sliced_kv_destroy(handle)
             self._handle = None
 
     def map_kernel_id(self) -> int:
