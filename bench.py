@@ -1,0 +1,399 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged GQA split-KV SDPA path on one MI355X.
+
+`python bench.py [--gpus 1] [--steps K] [--warmup W]` prints ONE JSON line.  A step is one pass of the
+hot path (Map + Reduce, or the direct Map) over one batch of synthetic input that already sits in HBM.
+The headline workload is BASELINE config 2 (32 ragged decode requests, 512-token split-KV partitions);
+the other synthetic configs are timed briefly and reported under "configs".
+
+Inputs: Q/K/V ~ N(0,1) rounded to bf16 (generated on the device, fixed seeds), context lengths and page
+permutations from numpy's PCG64 seeded with the config index.  KV pools rotate between steps (three
+distinct pools) so no pool stays resident in the 256 MB Infinity Cache: the HBM figure is a cold one.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+TOKENS_PER_PAGE = 16
+NUM_POOLS = 3
+
+CONFIGS = {
+    1: dict(name="config1: B=1 q=1 Hq32/Hkv8/D128 ctx 1024, identity pages", hq=32, hkv=8, d=128, kind="decode", kv_slice=64),
+    2: dict(name="config2: B=32 q=1 Hq64/Hkv8/D128 ctx U[512,8192], 20480-page pool, 512-token partitions + LSE reduce",
+            hq=64, hkv=8, d=128, kind="decode", kv_slice=512),
+    3: dict(name="config3: B=4 q=1 Hq24/Hkv4/D256 ctx 131072, 2048-token partitions, output x sigmoid(gate)",
+            hq=24, hkv=4, d=256, kind="decode", kv_slice=2048, gated=True),
+    4: dict(name="config4: B=16 spec-verify q=1+k (k in 1..4), ctx U[4096,32768], Hq64/Hkv8/D128", hq=64, hkv=8, d=128,
+            kind="verify"),
+    5: dict(name="config5: B=8 chunked prefill, 2048-token chunk on prefix U[0,16384], Hq64/Hkv8/D128", hq=64, hkv=8, d=128,
+            kind="prefill"),
+}
+
+
+def sample_lengths(index: int):
+    """(histories, q_lens) of a config; numpy PCG64 seeded with the config index."""
+    rng = np.random.default_rng(index)
+    if index == 1:
+        return [1023], [1]
+    if index == 2:
+        contexts = rng.integers(512, 8193, size=32)
+        return [int(c) - 1 for c in contexts], [1] * 32
+    if index == 3:
+        return [131071] * 4, [1] * 4
+    if index == 4:
+        prior = rng.integers(4096, 32769, size=16)
+        drafts = rng.integers(1, 5, size=16)
+        return [int(p) for p in prior], [1 + int(k) for k in drafts]
+    if index == 5:
+        prefix = rng.integers(0, 16385, size=8)
+        return [int(p) for p in prefix], [2048] * 8
+    raise ValueError(index)
+
+
+class Workload:
+    """One synthetic config resident in HBM plus its recorded launches."""
+
+    def __init__(self, index: int, device, num_pools: int = NUM_POOLS):
+        import torch
+
+        from khalamari_amd import batch_metadata, sdpa, sliced_kv, sliced_q
+        from khalamari_amd._lib import DTYPE_BF16, DTYPE_F32, ReplayU32
+        from khalamari_amd.selector import GQAReplayBucketPolicy, RequestShape, Selector
+
+        spec = CONFIGS[index]
+        self.index, self.spec, self.device = index, spec, device
+        hq, hkv, d = spec["hq"], spec["hkv"], spec["d"]
+        self.histories, self.q_lens = sample_lengths(index)
+        contexts = [h + n for h, n in zip(self.histories, self.q_lens)]
+        num_requests = len(contexts)
+        pages_per_request = [-(-c // TOKENS_PER_PAGE) for c in contexts]
+        pool_pages = max(sum(pages_per_request), 20480 if index == 2 else 0)
+        num_blocks = max(pages_per_request)
+        rng = np.random.default_rng(1000 + index)
+        order = np.arange(pool_pages) if index == 1 else rng.permutation(pool_pages)
+        table = np.zeros((num_requests, num_blocks), dtype=np.uint32)
+        cursor = 0
+        for r, n in enumerate(pages_per_request):
+            table[r, :n] = order[cursor:cursor + n]
+            cursor += n
+        self.page_bytes = 2 * hkv * TOKENS_PER_PAGE * d * 2
+        generator = torch.Generator(device=device)
+        generator.manual_seed(index)
+        self.kv_pools = [
+            torch.randn(pool_pages * self.page_bytes // 2, device=device, dtype=torch.float32, generator=generator).to(torch.bfloat16)
+            for _ in range(num_pools)
+        ]
+        self.num_tokens = sum(self.q_lens)
+        self.q = torch.randn((self.num_tokens, hq, d), device=device, dtype=torch.float32, generator=generator).to(torch.bfloat16)
+        self.gates = None
+        if spec.get("gated"):
+            self.gates = torch.randn((self.num_tokens, hq, d), device=device, dtype=torch.float32, generator=generator).to(torch.bfloat16)
+        self.page_table = torch.from_numpy(table.reshape(-1).view(np.int32)).to(device)
+        self.table_host = table
+        self.out = torch.zeros((self.num_tokens, hq, d), dtype=torch.bfloat16, device=device)
+
+        # prepare: selector -> metadata, as GQA::prepare does once per batch
+        layout = sliced_kv.Layout(num_requests, 1, num_blocks, 1)
+        sconfig = sdpa.Config(DTYPE_BF16, hq, hkv, d, TOKENS_PER_PAGE)
+        cu_tokens = [0]
+        for n in self.q_lens:
+            cu_tokens.append(cu_tokens[-1] + n)
+        shapes = RequestShape.from_batch(self.histories, cu_tokens)
+        ratio = hq // hkv
+        if spec["kind"] == "decode":
+            variant = sdpa.ExecutionVariant.sliced_kv(sconfig, d, 128, min(ratio, 8))
+            max_splits = max(-(-c // spec["kv_slice"]) for c in contexts)
+            selector = Selector.for_partitions(sdpa.Registry.from_variants(sconfig, [variant]), self.num_tokens, num_requests,
+                                               lambda v: max_splits)
+            limits = selector.limits()
+            policy = GQAReplayBucketPolicy(limits.max_tokens, limits.max_map_task_templates)
+            selection = selector.select_partitioned(variant, spec["kv_slice"], False, shapes, policy, self.num_tokens)
+        else:
+            selector = Selector.for_lookup(sconfig, self.num_tokens, layout)
+            limits = selector.limits()
+            policy = GQAReplayBucketPolicy(limits.max_tokens, limits.max_map_task_templates)
+            selection = selector.select(shapes, policy, self.num_tokens)
+        self.selection = selection
+        self.variant = selection.variant()
+        self.direct = selection.direct_output()
+        self.metadata = batch_metadata.GQAMetadataBuffers(limits.max_tokens, limits.max_map_task_templates)
+        shape = self.metadata.update(list(range(num_requests)), self.histories, cu_tokens, selection)
+        self.replay_shape = shape
+        self.visible_tokens = sum(contexts)
+        partial_dtype = DTYPE_F32 if os.environ.get("KHM_BENCH_PARTIAL", "bf16") == "f32" else DTYPE_BF16
+        fixed = ReplayU32.fixed
+        md = self.metadata
+        if self.variant.map_kind == sdpa.MAP_SLICED_KV:
+            config = sliced_kv.Config(hq, hkv, d, d ** -0.5, self.page_bytes, layout, DTYPE_BF16, DTYPE_BF16, partial_dtype)
+            kshape = sliced_kv.Shape(shape.num_total_tokens, shape.num_total_sdpa_map_task_templates)
+            compute = sliced_kv.Compute(config, self.variant, kshape)
+            scratch = sliced_kv.Scratch(device, config, kshape)
+            self._keep = (compute, scratch)
+
+            def launch_map(pool):
+                compute.invoke_map(q=self.q, kv_pages=pool, req_slots=md.req_slots(), page_ids=self.page_table,
+                                   sdpa_map_task_templates=md.sdpa_map_task_templates(), partial_exp_sums=scratch.partial_exp_sums,
+                                   partial_max_logits=scratch.partial_max_logits, partial_output=scratch.partial_output,
+                                   page_table_index=fixed(0), num_active_tokens=fixed(shape.num_tokens),
+                                   num_active_kv_splits=fixed(shape.num_sdpa_map_task_templates))
+
+            def launch_reduce():
+                compute.invoke_reduce(partial_exp_sums=scratch.partial_exp_sums, partial_max_logits=scratch.partial_max_logits,
+                                      partial_output=scratch.partial_output, cu_sdpa_partial_outputs=md.cu_sdpa_partial_outputs(),
+                                      output=self.out, num_active_tokens=fixed(shape.num_tokens), gates=self.gates)
+        else:
+            config = sliced_q.Config(hq, hkv, d, d ** -0.5, self.page_bytes, layout, DTYPE_BF16, DTYPE_BF16, partial_dtype)
+            qshape = sliced_q.Shape(shape.num_total_tokens, shape.num_total_q_token_tiles, shape.num_total_sdpa_map_task_templates)
+            common = dict(q=self.q, req_slots=md.req_slots(), page_ids=self.page_table,
+                          visible_kv_token_ranges=md.visible_kv_token_ranges(), q_token_ranges=md.q_token_ranges(),
+                          sdpa_map_task_templates=md.sdpa_map_task_templates(), page_table_index=fixed(0),
+                          num_active_tokens=fixed(shape.num_tokens), num_active_q_token_tiles=fixed(shape.num_q_token_tiles))
+            if self.direct:
+                compute = sliced_q.Compute.new_direct(config, self.variant, qshape)
+                self._keep = (compute,)
+
+                def launch_map(pool):
+                    compute.invoke_direct(kv_pages=pool, output=self.out, **common)
+
+                launch_reduce = None
+            else:
+                compute = sliced_q.Compute.new(config, self.variant, qshape)
+                partial = torch.zeros(config.partial_output_bytes(self.variant, qshape), dtype=torch.uint8, device=device)
+                sums = torch.zeros(config.partial_output_stats_bytes(self.variant, qshape), dtype=torch.uint8, device=device)
+                maxs = torch.zeros_like(sums)
+                self._keep = (compute, partial, sums, maxs)
+
+                def launch_map(pool):
+                    compute.invoke_map(kv_pages=pool, partial_output=partial, partial_exp_sums=sums, partial_max_logits=maxs,
+                                       num_active_kv_splits=fixed(shape.num_sdpa_map_task_templates), **common)
+
+                def launch_reduce():
+                    compute.invoke_reduce(partial_output=partial, partial_exp_sums=sums, partial_max_logits=maxs,
+                                          q_token_ranges=md.q_token_ranges(), cu_sdpa_partial_outputs=md.cu_sdpa_partial_outputs(),
+                                          output=self.out, num_active_q_token_tiles=fixed(shape.num_q_token_tiles))
+        self.launch_map, self.launch_reduce = launch_map, launch_reduce
+
+    # ---- algorithmic work ------------------------------------------------------------------------------
+    def algorithmic_bytes(self) -> int:
+        """K/V bytes of every visible token once per sequence, plus Q, output and page-table reads."""
+        spec = self.spec
+        kv = self.visible_tokens * spec["hkv"] * spec["d"] * 2 * 2
+        qo = 2 * self.num_tokens * spec["hq"] * spec["d"] * 2
+        table = sum(-(-(h + n) // TOKENS_PER_PAGE) for h, n in zip(self.histories, self.q_lens)) * 4
+        return kv + qo + table
+
+    def algorithmic_flops(self) -> int:
+        """4 * Hq * D * sum(C * P + C (C + 1) / 2): two GEMMs, causal-exact."""
+        spec = self.spec
+        pairs = sum(n * h + n * (n + 1) // 2 for h, n in zip(self.histories, self.q_lens))
+        return 4 * spec["hq"] * spec["d"] * pairs
+
+    def step(self, i: int) -> None:
+        self.launch_map(self.kv_pools[i % len(self.kv_pools)])
+        if self.launch_reduce is not None:
+            self.launch_reduce()
+
+    def time_steps(self, steps: int, warmup: int):
+        """(ms per step over a clean timed region, mean Map-kernel ms from per-launch HIP events)."""
+        import torch
+
+        for i in range(warmup):
+            self.step(i)
+        torch.cuda.synchronize()
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        begin.record()
+        for i in range(steps):
+            self.step(i)
+        end.record()
+        torch.cuda.synchronize()
+        ms_per_step = begin.elapsed_time(end) / steps
+        # per-kernel region: events on the launch stream around every Map launch
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for i, (a, b) in enumerate(pairs):
+            a.record()
+            self.launch_map(self.kv_pools[i % len(self.kv_pools)])
+            b.record()
+            if self.launch_reduce is not None:
+                self.launch_reduce()
+        torch.cuda.synchronize()
+        map_ms = sorted(a.elapsed_time(b) for a, b in pairs)
+        return ms_per_step, float(np.mean(map_ms)), float(map_ms[len(map_ms) // 2])
+
+    def report(self, steps: int, warmup: int) -> dict:
+        ms, map_ms, map_ms_median = self.time_steps(steps, warmup)
+        spec = self.spec
+        result = {
+            "workload": spec["name"],
+            "us_per_step": ms * 1e3,
+            "map_kernel_us": map_ms * 1e3,
+            "map_kernel_us_median": map_ms_median * 1e3,
+            "map_kind": int(self.variant.map_kind),
+            "map_tile": [int(self.variant.map_max_q_tokens), int(self.variant.map_max_q_heads)],
+            "direct_output": bool(self.direct),
+            "map_task_templates": int(self.replay_shape.num_sdpa_map_task_templates),
+            "visible_kv_tokens": int(self.visible_tokens),
+        }
+        if spec["kind"] == "prefill":
+            flops = self.algorithmic_flops()
+            result.update(bound="mfma", algorithmic_flops=flops, tflops=flops / (ms * 1e-3) / 1e12,
+                          map_tflops=flops / (map_ms * 1e-3) / 1e12)
+            result["roofline_frac"] = result["map_tflops"] / MFMA_BF16_PEAK_TFLOPS
+        else:
+            nbytes = self.algorithmic_bytes()
+            result.update(bound="hbm", algorithmic_bytes=nbytes, gbps=nbytes / (ms * 1e-3) / 1e9,
+                          map_gbps=nbytes / (map_ms * 1e-3) / 1e9)
+            result["roofline_frac"] = result["map_gbps"] / HBM_PEAK_GBPS
+        return result
+
+
+def cpu_baseline(index: int = 2, seconds_hint: float = 20.0) -> dict:
+    """Times the CPU oracle (a port of the reference's scalar f32 attention, gathering through the page table) on a
+    bounded sample of the headline workload: the shortest sequences of config 2 until about `seconds_hint` of
+    single-thread work is reached, once single-threaded and once on all host cores."""
+    from oracle import gqa_oracle as oracle
+
+    spec = CONFIGS[index]
+    histories, q_lens = sample_lengths(index)
+    order = np.argsort(histories)
+    hq, hkv, d = spec["hq"], spec["hkv"], spec["d"]
+    # about 0.25 G multiply-adds per second per thread for the strictly ordered scalar loops
+    budget_tokens = int(seconds_hint * 0.25e9 / (hq * d * 2))
+    chosen, total = [], 0
+    for r in order:
+        if chosen and total + histories[r] + 1 > budget_tokens:
+            break
+        chosen.append(int(r))
+        total += histories[r] + 1
+    rng = np.random.default_rng(7)
+    sample_hist = [histories[r] for r in chosen]
+    contexts = [h + 1 for h in sample_hist]
+    pages = [-(-c // TOKENS_PER_PAGE) for c in contexts]
+    geom = oracle.Geometry(hq, hkv, d, TOKENS_PER_PAGE, d ** -0.5, 1, max(pages), 1)
+    order_pages = rng.permutation(sum(pages))
+    table = np.zeros((len(chosen), max(pages)), dtype=np.uint32)
+    cursor = 0
+    for i, n in enumerate(pages):
+        table[i, :n] = order_pages[cursor:cursor + n]
+        cursor += n
+    kv = oracle.f32_to_bf16_bits(rng.standard_normal(sum(pages) * geom.page_bytes // 2, dtype=np.float32))
+    q = oracle.f32_to_bf16_bits(rng.standard_normal((len(chosen), hq, d), dtype=np.float32))
+    slots = np.arange(len(chosen), dtype=np.uint32)
+    visible = np.array([[0, c] for c in contexts], dtype=np.uint32)
+    nbytes = sum(contexts) * hkv * d * 4
+    timings = {}
+    threads = oracle.max_threads()
+    for label, n in (("single_thread", 1), ("all_cores", threads)):
+        start = time.perf_counter()
+        oracle.paged_gqa(geom, q, kv.view(np.uint8), slots, table.reshape(-1), visible, num_threads=n)
+        timings[label] = time.perf_counter() - start
+    return {
+        "value": nbytes / timings["all_cores"] / 1e9,
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"{len(chosen)} shortest of the 32 config-2 sequences ({sum(contexts)} KV tokens, {nbytes / 1e6:.1f} MB of K/V), "
+                  f"f32 C oracle, OpenMP over (token, KV head)",
+        "seconds": timings["all_cores"],
+        "single_thread_value": nbytes / timings["single_thread"] / 1e9,
+        "single_thread_seconds": timings["single_thread"],
+        "host_cpu": _cpu_model(),
+    }
+
+
+def _cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as handle:
+            for line in handle:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser(description=__doc__)
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=200)
+    parser.add_argument("--warmup", type=int, default=20)
+    parser.add_argument("--config", type=int, default=2, help="headline config (default 2)")
+    parser.add_argument("--only", action="store_true", help="time only the headline config (used for profiling runs)")
+    parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path shards by (sequence, KV head) with no exchange, and this build runs "
+              "on a single MI355X; rerun with --gpus 1", file=sys.stderr)
+        return 2
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X (no GPU visible)", file=sys.stderr)
+        return 2
+    device = torch.device("cuda:0")
+    headline = Workload(args.config, device)
+    head = headline.report(args.steps, args.warmup)
+    others = {}
+    if not args.only:
+        del headline
+        torch.cuda.empty_cache()
+        for index in sorted(CONFIGS):
+            if index == args.config:
+                continue
+            try:
+                workload = Workload(index, device)
+                others[f"config{index}"] = workload.report(max(args.steps // 4, 10), max(args.warmup // 2, 3))
+                del workload
+                torch.cuda.empty_cache()
+            except Exception as error:  # a config whose kernel is not built yet is reported, not hidden
+                others[f"config{index}"] = {"workload": CONFIGS[index]["name"], "error": str(error)}
+    prefill = head["bound"] == "mfma"
+    line = {
+        "metric": "paged GQA prefill bf16 MFMA TFLOP/s" if prefill else "paged GQA decode achieved HBM GB/s (Map + Reduce per step)",
+        "value": head["tflops"] if prefill else head["gbps"],
+        "unit": "TFLOP/s" if prefill else "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["us_per_step"] / 1e3,
+        "us_per_step": head["us_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": head["workload"], "kv_pools_rotated": NUM_POOLS, "map_task_templates": head["map_task_templates"],
+                   "visible_kv_tokens": head["visible_kv_tokens"]},
+        "roofline": {
+            "bound": head["bound"],
+            "achieved": head["map_tflops"] if prefill else head["map_gbps"],
+            "peak": MFMA_BF16_PEAK_TFLOPS if prefill else HBM_PEAK_GBPS,
+            "unit": "TFLOP/s" if prefill else "GB/s",
+            "frac": head["roofline_frac"],
+            "traffic": None,
+            "kernel": "split_kv_map_kernel",
+            "kernel_us": head["map_kernel_us"],
+            "algorithmic_bytes": head.get("algorithmic_bytes"),
+            "algorithmic_flops": head.get("algorithmic_flops"),
+        },
+        "configs": others,
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(2)
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
