@@ -135,6 +135,12 @@ class Workload:
         partial_dtype = DTYPE_F32 if os.environ.get("KHM_BENCH_PARTIAL", "bf16") == "f32" else DTYPE_BF16
         fixed = ReplayU32.fixed
         md = self.metadata
+        # Map and Reduce in one launch (the last block of a token merges) pays off when the step is launch-latency
+        # bound; large batches keep the two-launch form.  KHM_BENCH_FUSED=0/1 forces either.
+        choice = os.environ.get("KHM_BENCH_FUSED", "auto")
+        fused = choice == "1" or (choice == "auto" and self.visible_tokens * hkv * d * 4 < (64 << 20))
+        fused = fused and not self.direct
+        self.fused = fused
         if self.variant.map_kind == sdpa.MAP_SLICED_KV:
             config = sliced_kv.Config(hq, hkv, d, d ** -0.5, self.page_bytes, layout, DTYPE_BF16, DTYPE_BF16, partial_dtype)
             kshape = sliced_kv.Shape(shape.num_total_tokens, shape.num_total_sdpa_map_task_templates)
@@ -153,6 +159,22 @@ class Workload:
                 compute.invoke_reduce(partial_exp_sums=scratch.partial_exp_sums, partial_max_logits=scratch.partial_max_logits,
                                       partial_output=scratch.partial_output, cu_sdpa_partial_outputs=md.cu_sdpa_partial_outputs(),
                                       output=self.out, num_active_tokens=fixed(shape.num_tokens), gates=self.gates)
+
+            if fused:
+                counters = torch.zeros(compute.arrival_counters_bytes(), dtype=torch.uint8, device=device)
+                self._keep += (counters,)
+
+                def launch_map(pool):  # noqa: F811
+                    compute.invoke_map_reduce(q=self.q, kv_pages=pool, req_slots=md.req_slots(), page_ids=self.page_table,
+                                              sdpa_map_task_templates=md.sdpa_map_task_templates(),
+                                              partial_exp_sums=scratch.partial_exp_sums, partial_max_logits=scratch.partial_max_logits,
+                                              partial_output=scratch.partial_output,
+                                              cu_sdpa_partial_outputs=md.cu_sdpa_partial_outputs(), output=self.out,
+                                              arrival_counters=counters, page_table_index=fixed(0),
+                                              num_active_tokens=fixed(shape.num_tokens),
+                                              num_active_kv_splits=fixed(shape.num_sdpa_map_task_templates), gates=self.gates)
+
+                launch_reduce = None
         else:
             config = sliced_q.Config(hq, hkv, d, d ** -0.5, self.page_bytes, layout, DTYPE_BF16, DTYPE_BF16, partial_dtype)
             qshape = sliced_q.Shape(shape.num_total_tokens, shape.num_total_q_token_tiles, shape.num_total_sdpa_map_task_templates)
@@ -183,6 +205,18 @@ class Workload:
                     compute.invoke_reduce(partial_output=partial, partial_exp_sums=sums, partial_max_logits=maxs,
                                           q_token_ranges=md.q_token_ranges(), cu_sdpa_partial_outputs=md.cu_sdpa_partial_outputs(),
                                           output=self.out, num_active_q_token_tiles=fixed(shape.num_q_token_tiles))
+
+                if fused:
+                    counters = torch.zeros(compute.arrival_counters_bytes(), dtype=torch.uint8, device=device)
+                    self._keep += (counters,)
+
+                    def launch_map(pool):  # noqa: F811
+                        compute.invoke_map_reduce(kv_pages=pool, partial_output=partial, partial_exp_sums=sums, partial_max_logits=maxs,
+                                                  cu_sdpa_partial_outputs=md.cu_sdpa_partial_outputs(), output=self.out,
+                                                  arrival_counters=counters,
+                                                  num_active_kv_splits=fixed(shape.num_sdpa_map_task_templates), **common)
+
+                    launch_reduce = None
         self.launch_map, self.launch_reduce = launch_map, launch_reduce
 
     # ---- algorithmic work ------------------------------------------------------------------------------
@@ -242,6 +276,7 @@ class Workload:
             "map_kind": int(self.variant.map_kind),
             "map_tile": [int(self.variant.map_max_q_tokens), int(self.variant.map_max_q_heads)],
             "direct_output": bool(self.direct),
+            "fused_reduce": bool(self.fused),
             "map_task_templates": int(self.replay_shape.num_sdpa_map_task_templates),
             "visible_kv_tokens": int(self.visible_tokens),
         }
@@ -360,7 +395,7 @@ def main() -> int:
                 others[f"config{index}"] = {"workload": CONFIGS[index]["name"], "error": str(error)}
     prefill = head["bound"] == "mfma"
     line = {
-        "metric": "paged GQA prefill bf16 MFMA TFLOP/s" if prefill else "paged GQA decode achieved HBM GB/s (Map + Reduce per step)",
+        "metric": "paged GQA prefill bf16 MFMA TFLOP/s" if prefill else "paged GQA decode achieved HBM GB/s (split-KV Map + LSE Reduce per step)",
         "value": head["tflops"] if prefill else head["gbps"],
         "unit": "TFLOP/s" if prefill else "GB/s",
         "n_gpus": 1,

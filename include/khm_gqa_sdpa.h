@@ -217,6 +217,23 @@ int khm_sliced_kv_reduce_gated(const khm_sliced_kv* compute, const khm_sliced_kv
                                khm_buffer gates, khm_replay_u32 num_active_tokens,
                                const uint32_t* replay_parameters, void* stream);
 
+/* Map and Reduce in one launch.  The reference records two operators with a barrier between them
+ * (attn/gqa/backend.rs:458-482); on gfx950 the second launch and its dependent loads cost several
+ * microseconds of a ~100 us decode step, so the last Map block to finish a (token, KV head) merges that
+ * token's partial states itself.  Same partial buffers and merge formula as khm_sliced_kv_map followed by
+ * khm_sliced_kv_reduce[_gated]; only the summation order of the merge differs.
+ *   arrival_counters  u32 [num_total_tokens][Hkv * q_head_ranges], all zero before the first launch; every
+ *                     launch leaves them zero again, so one memset at allocation is enough.  Launches that
+ *                     share the counters must not overlap.
+ *   gates             optional (ptr == NULL: no gate). */
+uint64_t khm_sliced_kv_arrival_counters_bytes(const khm_gqa_sdpa_config* config, const khm_sdpa_variant* variant,
+                                              const khm_gqa_sdpa_shape* shape);
+int khm_sliced_kv_map_reduce(const khm_sliced_kv* compute, const khm_sliced_kv_map_buffers* map_buffers,
+                             const khm_sliced_kv_reduce_buffers* reduce_buffers, khm_buffer gates,
+                             khm_buffer arrival_counters, khm_replay_u32 page_table_index,
+                             khm_replay_u32 num_active_tokens, khm_replay_u32 num_active_kv_splits,
+                             const uint32_t* replay_parameters, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Sliced-Q component: sdpa/sliced_q.rs (verify blocks and chunked prefill)
  * ------------------------------------------------------------------------------------------ */
@@ -282,6 +299,16 @@ int khm_sliced_q_direct(const khm_sliced_q* compute, const khm_sliced_q_direct_b
 /* Compute::invoke_reduce + ReduceInvocation::record (sliced_q.rs:484-504,620-642). */
 int khm_sliced_q_reduce(const khm_sliced_q* compute, const khm_sliced_q_reduce_buffers* buffers,
                         khm_replay_u32 num_active_q_token_tiles, const uint32_t* replay_parameters, void* stream);
+
+/* Map and Reduce in one launch for the sliced-Q component; see khm_sliced_kv_map_reduce.
+ *   arrival_counters  u32 [num_total_q_token_tiles][Hkv * q_head_ranges], zero before the first launch. */
+uint64_t khm_sliced_q_arrival_counters_bytes(const khm_gqa_sdpa_config* config, const khm_sdpa_variant* variant,
+                                             const khm_gqa_sdpa_shape* shape);
+int khm_sliced_q_map_reduce(const khm_sliced_q* compute, const khm_sliced_q_map_buffers* map_buffers,
+                            const khm_sliced_q_reduce_buffers* reduce_buffers, khm_buffer arrival_counters,
+                            khm_replay_u32 page_table_index, khm_replay_u32 num_active_tokens,
+                            khm_replay_u32 num_active_q_token_tiles, khm_replay_u32 num_active_kv_splits,
+                            const uint32_t* replay_parameters, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Sigmoid gate: components/gqa/activation_gate.rs:35-168, gqa_activation_gate.metal:14-59

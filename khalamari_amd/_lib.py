@@ -9,7 +9,7 @@ import ctypes
 import os
 
 _PACKAGE_DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PACKAGE_DIR, "lib", "libkhm_gqa_sdpa.so")
+LIB_PATH = os.environ.get("KHM_LIB_PATH") or os.path.join(_PACKAGE_DIR, "lib", "libkhm_gqa_sdpa.so")
 
 KHM_OK = 0
 KHM_ERR_INVALID_ARGUMENT = -1
@@ -172,9 +172,10 @@ EXPORTED_SYMBOLS = (
     "khm_gqa_sdpa_num_tokens_per_page", "khm_gqa_sdpa_q_bytes", "khm_gqa_sdpa_page_ids_bytes",
     "khm_sliced_kv_partial_output_stats_bytes", "khm_sliced_kv_partial_output_bytes", "khm_sliced_kv_create",
     "khm_sliced_kv_destroy", "khm_sliced_kv_map_kernel_id", "khm_sliced_kv_reduce_kernel_id", "khm_sliced_kv_map",
-    "khm_sliced_kv_reduce", "khm_sliced_kv_reduce_gated",
+    "khm_sliced_kv_reduce", "khm_sliced_kv_reduce_gated", "khm_sliced_kv_arrival_counters_bytes", "khm_sliced_kv_map_reduce",
     "khm_sliced_q_partial_output_bytes", "khm_sliced_q_partial_output_stats_bytes", "khm_sliced_q_create",
     "khm_sliced_q_destroy", "khm_sliced_q_map_kernel_id", "khm_sliced_q_map", "khm_sliced_q_direct", "khm_sliced_q_reduce",
+    "khm_sliced_q_arrival_counters_bytes", "khm_sliced_q_map_reduce",
     "khm_gqa_activation_gate",
     "khm_bf16_to_fp8_e4m3", "khm_fp8_e4m3_to_bf16", "khm_f32_to_bf16", "khm_bf16_to_f32",
     "khm_replay_bucket_policy_create", "khm_replay_bucket_policy_destroy", "khm_replay_bucket_policy_max_capacity",
@@ -212,7 +213,8 @@ def lib() -> ctypes.CDLL:
     handle.khm_version.restype = ctypes.c_char_p
     for name in ("khm_gqa_sdpa_q_bytes", "khm_gqa_sdpa_page_ids_bytes", "khm_sliced_kv_partial_output_stats_bytes",
                  "khm_sliced_kv_partial_output_bytes", "khm_sliced_q_partial_output_bytes",
-                 "khm_sliced_q_partial_output_stats_bytes"):
+                 "khm_sliced_q_partial_output_stats_bytes", "khm_sliced_kv_arrival_counters_bytes",
+                 "khm_sliced_q_arrival_counters_bytes"):
         getattr(handle, name).restype = u64
     handle.khm_gqa_sdpa_num_tokens_per_page.restype = u32
     for name in ("khm_sliced_kv_map_kernel_id", "khm_sliced_kv_reduce_kernel_id", "khm_sliced_q_map_kernel_id"):
@@ -235,6 +237,12 @@ def lib() -> ctypes.CDLL:
                                             ctypes.c_void_p]
     handle.khm_sliced_kv_reduce_gated.argtypes = [ctypes.c_void_p, ctypes.POINTER(SlicedKvReduceBuffers), Buffer, ReplayU32,
                                                   ctypes.c_void_p, ctypes.c_void_p]
+    handle.khm_sliced_kv_map_reduce.argtypes = [ctypes.c_void_p, ctypes.POINTER(SlicedKvMapBuffers),
+                                                ctypes.POINTER(SlicedKvReduceBuffers), Buffer, Buffer, ReplayU32, ReplayU32, ReplayU32,
+                                                ctypes.c_void_p, ctypes.c_void_p]
+    handle.khm_sliced_q_map_reduce.argtypes = [ctypes.c_void_p, ctypes.POINTER(SlicedQMapBuffers),
+                                               ctypes.POINTER(SlicedQReduceBuffers), Buffer, ReplayU32, ReplayU32, ReplayU32, ReplayU32,
+                                               ctypes.c_void_p, ctypes.c_void_p]
     handle.khm_sliced_q_map.argtypes = [ctypes.c_void_p, ctypes.POINTER(SlicedQMapBuffers), ReplayU32, ReplayU32, ReplayU32,
                                         ReplayU32, ctypes.c_void_p, ctypes.c_void_p]
     handle.khm_sliced_q_direct.argtypes = [ctypes.c_void_p, ctypes.POINTER(SlicedQDirectBuffers), ReplayU32, ReplayU32,

@@ -37,11 +37,11 @@ HIPCC_FLAGS = [
 ]
 
 
-def build(verbose: bool = False, extra_flags=()) -> str:
+def build(verbose: bool = False, extra_flags=(), output: str = LIB_PATH) -> str:
     os.makedirs(LIB_DIR, exist_ok=True)
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     sources = [os.path.join(CSRC_DIR, name) for name in SOURCES if os.path.exists(os.path.join(CSRC_DIR, name))]
-    command = [hipcc, *HIPCC_FLAGS, *extra_flags, "-x", "hip", *sources, "-o", LIB_PATH]
+    command = [hipcc, *HIPCC_FLAGS, *extra_flags, "-x", "hip", *sources, "-o", output]
     if verbose:
         print(" ".join(command), flush=True)
     result = subprocess.run(command, capture_output=True, text=True)
@@ -51,7 +51,7 @@ def build(verbose: bool = False, extra_flags=()) -> str:
         raise RuntimeError(f"hipcc failed ({result.returncode}):\n{stderr}")
     if verbose and stderr.strip():
         print(stderr, file=sys.stderr)
-    return LIB_PATH
+    return output
 
 
 if __name__ == "__main__":

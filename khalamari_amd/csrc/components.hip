@@ -12,7 +12,10 @@
 
 namespace khm {
 
-constexpr int kMapWaves = 4;
+#ifndef KHM_MAP_WAVES
+#define KHM_MAP_WAVES 4
+#endif
+constexpr int kMapWaves = KHM_MAP_WAVES;
 
 typedef void (*MapKernel)(const MapParams);
 typedef void (*ReduceKernel)(const ReduceParams);
@@ -228,10 +231,17 @@ extern "C" const void* khm_sliced_kv_reduce_kernel_id(const khm_sliced_kv* compu
     return reinterpret_cast<const void*>(compute->reduce);
 }
 
-extern "C" int khm_sliced_kv_map(const khm_sliced_kv* compute, const khm_sliced_kv_map_buffers* buffers,
-                                 khm_replay_u32 page_table_index, khm_replay_u32 num_active_tokens,
-                                 khm_replay_u32 num_active_kv_splits, const uint32_t* replay_parameters, void* stream) {
-    clear_error();
+struct FusedReduceArgs {
+    const uint32_t* cu_partial_outputs;
+    uint32_t* arrival_counters;
+    uint16_t* final_output;
+    const uint16_t* gates;
+};
+
+static int launch_sliced_kv_map(const khm_sliced_kv* compute, const khm_sliced_kv_map_buffers* buffers,
+                                khm_replay_u32 page_table_index, khm_replay_u32 num_active_tokens,
+                                khm_replay_u32 num_active_kv_splits, const uint32_t* replay_parameters, void* stream,
+                                const FusedReduceArgs* fused) {
     KHM_REQUIRE(compute != nullptr && buffers != nullptr, "compute and buffers must not be null");
     const khm_gqa_sdpa_config& config = compute->config;
     const khm_gqa_sdpa_shape& shape = compute->shape;
@@ -266,9 +276,52 @@ extern "C" int khm_sliced_kv_map(const khm_sliced_kv* compute, const khm_sliced_
     p.num_active_kv_splits = to_device(num_active_kv_splits);
     fill_map_geometry(*compute, &p);
     p.output_mode = config.partial_dtype == KHM_DTYPE_F32 ? kMapPartialF32 : kMapPartialBf16;
+    if (fused != nullptr) {
+        p.cu_partial_outputs = fused->cu_partial_outputs;
+        p.arrival_counters = fused->arrival_counters;
+        p.final_output = fused->final_output;
+        p.gates = fused->gates;
+    }
     const dim3 grid(shape.num_total_sdpa_map_task_templates, config.num_kv_heads * compute->num_q_head_ranges, 1);
     hipLaunchKernelGGL(compute->map, grid, dim3(kMapWaves * 64), 0, static_cast<hipStream_t>(stream), p);
     return check_launch("sliced-KV map");
+}
+
+extern "C" int khm_sliced_kv_map(const khm_sliced_kv* compute, const khm_sliced_kv_map_buffers* buffers,
+                                 khm_replay_u32 page_table_index, khm_replay_u32 num_active_tokens,
+                                 khm_replay_u32 num_active_kv_splits, const uint32_t* replay_parameters, void* stream) {
+    clear_error();
+    return launch_sliced_kv_map(compute, buffers, page_table_index, num_active_tokens, num_active_kv_splits, replay_parameters, stream,
+                                nullptr);
+}
+
+extern "C" uint64_t khm_sliced_kv_arrival_counters_bytes(const khm_gqa_sdpa_config* config, const khm_sdpa_variant* variant,
+                                                         const khm_gqa_sdpa_shape* shape) {
+    const uint32_t ranges = div_ceil_u32(config->num_q_heads / config->num_kv_heads, variant->map_max_q_heads);
+    return (uint64_t)shape->num_total_tokens * config->num_kv_heads * ranges * 4;
+}
+
+extern "C" int khm_sliced_kv_map_reduce(const khm_sliced_kv* compute, const khm_sliced_kv_map_buffers* map_buffers,
+                                        const khm_sliced_kv_reduce_buffers* reduce_buffers, khm_buffer gates, khm_buffer arrival_counters,
+                                        khm_replay_u32 page_table_index, khm_replay_u32 num_active_tokens,
+                                        khm_replay_u32 num_active_kv_splits, const uint32_t* replay_parameters, void* stream) {
+    clear_error();
+    KHM_REQUIRE(compute != nullptr && map_buffers != nullptr && reduce_buffers != nullptr, "compute and buffers must not be null");
+    const khm_gqa_sdpa_config& config = compute->config;
+    const khm_gqa_sdpa_shape& shape = compute->shape;
+    KHM_REQUIRE(reduce_buffers->partial_output.ptr == map_buffers->partial_output.ptr &&
+                    reduce_buffers->partial_exp_sums.ptr == map_buffers->partial_exp_sums.ptr &&
+                    reduce_buffers->partial_max_logits.ptr == map_buffers->partial_max_logits.ptr,
+                "fused Map/Reduce needs the same partial buffers on both sides");
+    KHM_BUFFER_AT_LEAST(reduce_buffers->cu_sdpa_partial_outputs, ((uint64_t)shape.num_total_tokens + 1) * 4, "cu_sdpa_partial_outputs");
+    KHM_BUFFER_AT_LEAST(reduce_buffers->output, khm_gqa_sdpa_q_bytes(&config, &shape), "output");
+    KHM_BUFFER_AT_LEAST(arrival_counters, khm_sliced_kv_arrival_counters_bytes(&config, &compute->variant, &shape), "arrival_counters");
+    if (gates.ptr != nullptr) KHM_BUFFER_AT_LEAST(gates, khm_gqa_sdpa_q_bytes(&config, &shape), "gates");
+    const FusedReduceArgs fused{static_cast<const uint32_t*>(reduce_buffers->cu_sdpa_partial_outputs.ptr),
+                                static_cast<uint32_t*>(arrival_counters.ptr), static_cast<uint16_t*>(reduce_buffers->output.ptr),
+                                static_cast<const uint16_t*>(gates.ptr)};
+    return launch_sliced_kv_map(compute, map_buffers, page_table_index, num_active_tokens, num_active_kv_splits, replay_parameters,
+                                stream, &fused);
 }
 
 static int launch_sliced_kv_reduce(const khm_sliced_kv* compute, const khm_sliced_kv_reduce_buffers* buffers, const khm_buffer* gates,
@@ -364,7 +417,8 @@ static int launch_sliced_q_map(const khm_sliced_q* compute, const khm_buffer& q,
                                const khm_buffer& templates, const khm_buffer* partial, const khm_buffer* sums,
                                const khm_buffer* maxs, const khm_buffer* output, khm_replay_u32 page_table_index,
                                khm_replay_u32 num_active_tokens, khm_replay_u32 num_active_q_token_tiles,
-                               khm_replay_u32 num_active_kv_splits, const uint32_t* replay_parameters, void* stream) {
+                               khm_replay_u32 num_active_kv_splits, const uint32_t* replay_parameters, void* stream,
+                               const FusedReduceArgs* fused = nullptr) {
     const khm_gqa_sdpa_config& config = compute->config;
     const khm_gqa_sdpa_shape& shape = compute->shape;
     // MapInvocation::validate / DirectInvocation::validate (sliced_q.rs:519-545)
@@ -406,9 +460,48 @@ static int launch_sliced_q_map(const khm_sliced_q* compute, const khm_buffer& q,
     p.num_active_q_token_tiles = to_device(num_active_q_token_tiles);
     p.num_active_kv_splits = to_device(num_active_kv_splits);
     fill_map_geometry(*compute, &p);
+    if (fused != nullptr) {
+        p.cu_partial_outputs = fused->cu_partial_outputs;
+        p.arrival_counters = fused->arrival_counters;
+        p.final_output = fused->final_output;
+        p.gates = fused->gates;
+    }
     const dim3 grid(shape.num_total_sdpa_map_task_templates, config.num_kv_heads * compute->num_q_head_ranges, 1);
     hipLaunchKernelGGL(compute->map, grid, dim3(kMapWaves * 64), 0, static_cast<hipStream_t>(stream), p);
     return check_launch("sliced-Q map");
+}
+
+extern "C" uint64_t khm_sliced_q_arrival_counters_bytes(const khm_gqa_sdpa_config* config, const khm_sdpa_variant* variant,
+                                                        const khm_gqa_sdpa_shape* shape) {
+    const uint32_t ranges = div_ceil_u32(config->num_q_heads / config->num_kv_heads, variant->map_max_q_heads);
+    return (uint64_t)shape->num_total_q_token_tiles * config->num_kv_heads * ranges * 4;
+}
+
+extern "C" int khm_sliced_q_map_reduce(const khm_sliced_q* compute, const khm_sliced_q_map_buffers* map_buffers,
+                                       const khm_sliced_q_reduce_buffers* reduce_buffers, khm_buffer arrival_counters,
+                                       khm_replay_u32 page_table_index, khm_replay_u32 num_active_tokens,
+                                       khm_replay_u32 num_active_q_token_tiles, khm_replay_u32 num_active_kv_splits,
+                                       const uint32_t* replay_parameters, void* stream) {
+    clear_error();
+    KHM_REQUIRE(compute != nullptr && map_buffers != nullptr && reduce_buffers != nullptr, "compute and buffers must not be null");
+    KHM_REQUIRE(!compute->direct, "GQA SplitKV SlicedQ direct-output compute cannot record a partial Map");
+    const khm_gqa_sdpa_config& config = compute->config;
+    const khm_gqa_sdpa_shape& shape = compute->shape;
+    KHM_REQUIRE(reduce_buffers->partial_output.ptr == map_buffers->partial_output.ptr &&
+                    reduce_buffers->partial_exp_sums.ptr == map_buffers->partial_exp_sums.ptr &&
+                    reduce_buffers->partial_max_logits.ptr == map_buffers->partial_max_logits.ptr &&
+                    reduce_buffers->q_token_ranges.ptr == map_buffers->q_token_ranges.ptr,
+                "fused Map/Reduce needs the same partial and Q-token-range buffers on both sides");
+    KHM_BUFFER_AT_LEAST(reduce_buffers->cu_sdpa_partial_outputs, ((uint64_t)shape.num_total_q_token_tiles + 1) * 4, "cu_sdpa_partial_outputs");
+    KHM_BUFFER_AT_LEAST(reduce_buffers->output, khm_gqa_sdpa_q_bytes(&config, &shape), "output");
+    KHM_BUFFER_AT_LEAST(arrival_counters, khm_sliced_q_arrival_counters_bytes(&config, &compute->variant, &shape), "arrival_counters");
+    const FusedReduceArgs fused{static_cast<const uint32_t*>(reduce_buffers->cu_sdpa_partial_outputs.ptr),
+                                static_cast<uint32_t*>(arrival_counters.ptr), static_cast<uint16_t*>(reduce_buffers->output.ptr), nullptr};
+    return launch_sliced_q_map(compute, map_buffers->q, map_buffers->kv_pages, map_buffers->req_slots, map_buffers->page_ids,
+                               map_buffers->visible_kv_token_ranges, map_buffers->q_token_ranges, map_buffers->sdpa_map_task_templates,
+                               &map_buffers->partial_output, &map_buffers->partial_exp_sums, &map_buffers->partial_max_logits, nullptr,
+                               page_table_index, num_active_tokens, num_active_q_token_tiles, num_active_kv_splits, replay_parameters,
+                               stream, &fused);
 }
 
 extern "C" int khm_sliced_q_map(const khm_sliced_q* compute, const khm_sliced_q_map_buffers* buffers, khm_replay_u32 page_table_index,

@@ -1,0 +1,69 @@
+// Small device helpers shared by the gfx950 kernels: vector typedefs, bf16 packing, exp2, the replay-parameter
+// resolver and the sigmoid used by the gate (gqa_activation_gate.metal:14-26 of the reference).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "device_params.h"
+
+namespace khm {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t resolve_u32(DeviceReplayU32 r, const uint32_t* params) {
+    return r.is_parameter ? params[r.value] : r.value;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+// e^x through v_exp_f32; both Reduce implementations use this one so they agree bit for bit.
+__device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits) { return __uint_as_float(bits << 16); }
+
+// Round-to-nearest-even f32 -> bf16 bits (v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float v) { return (uint16_t)(pack_bf16x2(v, 0.0f) & 0xffffu); }
+
+// Device-coherent accesses for data that another block on another XCD produces or consumes within one kernel:
+// relaxed agent-scope atomics compile to sc1 loads/stores that are served by memory instead of this XCD's
+// L2, so no cache write-back or invalidate is needed around them.
+__device__ __forceinline__ void coherent_store_u64(void* address, uint64_t value) {
+    __hip_atomic_store(reinterpret_cast<uint64_t*>(address), value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void coherent_store_f32(float* address, float value) {
+    __hip_atomic_store(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t coherent_load_u64(const void* address) {
+    return __hip_atomic_load(reinterpret_cast<const uint64_t*>(address), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float coherent_load_f32(const float* address) {
+    return __hip_atomic_load(address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ float round_to_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+
+// gqa_activation_gate.metal:19-26: sigmoid with every step rounded to bf16.
+__device__ __forceinline__ float sigmoid_bf16_steps(float x) {
+    const float abs_x = round_to_bf16(fabsf(x));
+    const float neg_abs_x = round_to_bf16(-abs_x);
+    const float exp_x = round_to_bf16(__expf(neg_abs_x));
+    const float denom = round_to_bf16(1.0f + exp_x);
+    const float y = round_to_bf16(1.0f / denom);
+    return x < 0.0f ? round_to_bf16(1.0f - y) : y;
+}
+
+// gqa_activation_gate.metal:14-17.
+__device__ __forceinline__ float sigmoid_f32(float x) {
+    const float y = 1.0f / (1.0f + __expf(-fabsf(x)));
+    return x < 0.0f ? 1.0f - y : y;
+}
+
+}  // namespace khm

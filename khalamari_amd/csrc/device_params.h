@@ -46,6 +46,11 @@ struct MapParams {
     uint32_t pages_per_request_layer;    // num_blocks * num_page_ids_per_block
     uint32_t output_mode;                // MapOutputMode
     float scale_log2e;                   // scale * log2(e)
+    // Fused Reduce (optional): the last block to finish a (Q range, head group) merges its partials.
+    const uint32_t* cu_partial_outputs;  // [R + 1]
+    uint32_t* arrival_counters;          // [R][gridDim.y], zero before the first launch; the merging block re-arms its counter
+    uint16_t* final_output;              // bf16 [T][Hq][D]
+    const uint16_t* gates;               // bf16 [T][Hq][D] or nullptr
 };
 
 // Arguments of the flat (sliced-KV) and ranged (sliced-Q) Reduce kernels.

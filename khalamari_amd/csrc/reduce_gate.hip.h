@@ -17,28 +17,11 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "device_math.hip.h"
 #include "device_params.h"
-#include "split_kv_map.hip.h"
+#include "lse_merge.hip.h"
 
 namespace khm {
-
-__device__ __forceinline__ float round_to_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
-
-// gqa_activation_gate.metal:19-26: sigmoid with every step rounded to bf16.
-__device__ __forceinline__ float sigmoid_bf16_steps(float x) {
-    const float abs_x = round_to_bf16(fabsf(x));
-    const float neg_abs_x = round_to_bf16(-abs_x);
-    const float exp_x = round_to_bf16(__expf(neg_abs_x));
-    const float denom = round_to_bf16(1.0f + exp_x);
-    const float y = round_to_bf16(1.0f / denom);
-    return x < 0.0f ? round_to_bf16(1.0f - y) : y;
-}
-
-// gqa_activation_gate.metal:14-17.
-__device__ __forceinline__ float sigmoid_f32(float x) {
-    const float y = 1.0f / (1.0f + __expf(-fabsf(x)));
-    return x < 0.0f ? 1.0f - y : y;
-}
 
 constexpr int kReduceThreads = 256;
 
@@ -48,9 +31,8 @@ template <int D, bool RANGED>
 __global__ __launch_bounds__(kReduceThreads) void split_kv_reduce_kernel(const ReduceParams p) {
     constexpr int CHUNKS = D / 4;                    // threads per row
     constexpr int SLICES = kReduceThreads / CHUNKS;  // partial slices per block
-    __shared__ float slice_max[SLICES];
-    __shared__ float slice_sum[SLICES];
-    __shared__ __align__(16) float slice_acc[SLICES][D];
+    __shared__ float slice_stats[SLICES * 2];
+    __shared__ __align__(16) float slice_acc[SLICES * D];
 
     const uint32_t unit = blockIdx.x;
     if (unit >= resolve_u32(p.num_active, p.replay_parameters)) return;
@@ -65,66 +47,24 @@ __global__ __launch_bounds__(kReduceThreads) void split_kv_reduce_kernel(const R
         if (num_q > max_q) num_q = max_q;
     }
     const int chunk = threadIdx.x % CHUNKS;
-    const int slice = threadIdx.x / CHUNKS;
+    const uint32_t slice = threadIdx.x / CHUNKS;
 
     for (uint32_t local = 0; local < num_q; ++local) {
-        float local_max = -INFINITY;
-        for (uint32_t part = begin + slice; part < end; part += SLICES) {
-            const uint64_t state = ((uint64_t)part * p.num_q_heads + head) * max_q + local;
-            local_max = fmaxf(local_max, p.max_logits[state]);
-        }
-        float local_sum = 0.0f;
-        f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-        for (uint32_t part = begin + slice; part < end; part += SLICES) {
-            const uint64_t state = ((uint64_t)part * p.num_q_heads + head) * max_q + local;
-            const float part_sum = p.exp_sums[state];
-            const float part_max = p.max_logits[state];
-            // sliced-KV guards on isfinite(max), sliced-Q on sum == 0; both describe the empty partial.
-            const bool empty = RANGED ? (part_sum == 0.0f) : !(fabsf(part_max) < INFINITY);
-            const float weight = empty ? 0.0f : __expf(part_max - local_max) * part_sum;
-            local_sum += weight;
-            f32x4 value;
-            if (p.partial_is_f32) {
-                value = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(p.partial) + state * D + chunk * 4);
-            } else {
-                const uint2 bits = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(p.partial) + state * D + chunk * 4);
-                value = f32x4{bf16_bits_to_f32(bits.x & 0xffffu), bf16_bits_to_f32(bits.x >> 16),
-                              bf16_bits_to_f32(bits.y & 0xffffu), bf16_bits_to_f32(bits.y >> 16)};
-            }
-            if (weight != 0.0f) acc += value * weight;
+        MergeState state = merge_state_empty();
+        if (end > begin) {
+            merge_partial_slice<D, false>(state, p.max_logits, p.exp_sums, p.partial, p.partial_is_f32 != 0, begin + slice, end, SLICES, begin,
+                                          p.num_q_heads, head, max_q, local, chunk);
         }
         if (chunk == 0) {
-            slice_max[slice] = local_max;
-            slice_sum[slice] = local_sum;
+            slice_stats[slice * 2] = state.run_max;
+            slice_stats[slice * 2 + 1] = state.run_sum;
         }
-        *reinterpret_cast<f32x4*>(&slice_acc[slice][chunk * 4]) = acc;
+        *reinterpret_cast<f32x4*>(slice_acc + slice * D + chunk * 4) = state.acc;
         __syncthreads();
         if (slice == 0) {
-            float global_max = -INFINITY;
-#pragma unroll
-            for (int s = 0; s < SLICES; ++s) global_max = fmaxf(global_max, slice_max[s]);
-            float global_sum = 0.0f;
-            f32x4 total = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-            for (int s = 0; s < SLICES; ++s) {
-                if (slice_sum[s] > 0.0f) {
-                    const float factor = __expf(slice_max[s] - global_max);
-                    global_sum += slice_sum[s] * factor;
-                    total += *reinterpret_cast<const f32x4*>(&slice_acc[s][chunk * 4]) * factor;
-                }
-            }
-            f32x4 result = {0.0f, 0.0f, 0.0f, 0.0f};
-            if (global_sum > 0.0f) result = total / global_sum;
+            const MergeState total = merge_combine_slices<D>(slice_stats, slice_acc, 0, SLICES, chunk);
             const uint64_t out_index = ((uint64_t)(flat_begin + local) * p.num_q_heads + head) * D + chunk * 4;
-            if (p.gates != nullptr) {
-                const uint2 gate_bits = *reinterpret_cast<const uint2*>(p.gates + out_index);
-                const float gate[4] = {bf16_bits_to_f32(gate_bits.x & 0xffffu), bf16_bits_to_f32(gate_bits.x >> 16),
-                                       bf16_bits_to_f32(gate_bits.y & 0xffffu), bf16_bits_to_f32(gate_bits.y >> 16)};
-#pragma unroll
-                for (int i = 0; i < 4; ++i) result[i] = round_to_bf16(result[i]) * sigmoid_bf16_steps(gate[i]);
-            }
-            const uint2 packed = make_uint2(pack_bf16x2(result[0], result[1]), pack_bf16x2(result[2], result[3]));
-            *reinterpret_cast<uint2*>(p.output + out_index) = packed;
+            merge_store_output(total, p.output, p.gates, out_index);
         }
         __syncthreads();
     }

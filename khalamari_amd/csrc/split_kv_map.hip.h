@@ -26,31 +26,11 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "device_math.hip.h"
 #include "device_params.h"
+#include "lse_merge.hip.h"
 
 namespace khm {
-
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ uint32_t resolve_u32(DeviceReplayU32 r, const uint32_t* params) {
-    return r.is_parameter ? params[r.value] : r.value;
-}
-
-__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-    f32x2 v = {lo, hi};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
-}
-
-__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits) { return __uint_as_float(bits << 16); }
-
-// Round-to-nearest-even f32 -> bf16 bits (v_cvt_pk_bf16_f32 on gfx950).
-__device__ __forceinline__ uint16_t f32_to_bf16_bits(float v) { return (uint16_t)(pack_bf16x2(v, 0.0f) & 0xffffu); }
 
 template <int D>
 struct KvTile {
@@ -73,8 +53,17 @@ struct MapSmem {
     static constexpr int kTotal = kUnionBytes + kQBytes + kStatsBytes;
 };
 
+#ifndef KHM_MAP_PREFETCH
+#define KHM_MAP_PREFETCH 2
+#endif
+#ifdef KHM_MAP_WAVES_PER_EU
+#define KHM_MAP_OCCUPANCY __attribute__((amdgpu_waves_per_eu(KHM_MAP_WAVES_PER_EU, KHM_MAP_WAVES_PER_EU)))
+#else
+#define KHM_MAP_OCCUPANCY
+#endif
+
 template <int D, int NT, int NWAVES>
-__global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapParams p) {
+__global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_kernel(const MapParams p) {
     constexpr int KS = D / 32;
     constexpr int MT = D / 16;
     constexpr int COLS = NT * 16;
@@ -97,7 +86,8 @@ __global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapPara
 
     // ---- task decode (uniform) -------------------------------------------------------------
     const uint32_t task = blockIdx.x;
-    if (task >= resolve_u32(p.num_active_kv_splits, p.replay_parameters)) return;
+    const uint32_t num_active_splits = resolve_u32(p.num_active_kv_splits, p.replay_parameters);
+    if (task >= num_active_splits) return;
     const uint32_t range_index = p.templates[3 * (uint64_t)task];
     if (range_index >= resolve_u32(p.num_active_q_token_tiles, p.replay_parameters)) return;
     uint32_t flat_begin, flat_end;
@@ -377,6 +367,7 @@ __global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapPara
 
     // ---- main loop: three rotating register buffers, loads two tiles ahead -----------------
     if (num_wave_tiles > 0) {
+#if KHM_MAP_PREFETCH == 2
         KvTile<D> t0, t1, t2;
         load_tile(0, t0);
         if (num_wave_tiles > 1) load_tile(1, t1);
@@ -392,6 +383,19 @@ __global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapPara
             compute_tile(t2);
             if (++j >= num_wave_tiles) break;
         }
+#else
+        KvTile<D> t0, t1;
+        load_tile(0, t0);
+        uint32_t j = 0;
+        while (true) {
+            if (j + 1 < num_wave_tiles) load_tile(j + 1, t1);
+            compute_tile(t0);
+            if (++j >= num_wave_tiles) break;
+            if (j + 1 < num_wave_tiles) load_tile(j + 1, t0);
+            compute_tile(t1);
+            if (++j >= num_wave_tiles) break;
+        }
+#endif
     }
 
     // ---- merge the waves of the block ------------------------------------------------------
@@ -443,6 +447,7 @@ __global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapPara
 
     // ---- write the block's partial state or final output ------------------------------------
     const uint32_t mode = p.output_mode;
+    const bool fused = p.arrival_counters != nullptr && mode != kMapDirectBf16;
     for (int index = tid; index < COLS * (D / 4); index += NWAVES * 64) {
         const uint32_t c = index / (D / 4);
         const uint32_t d = (index - c * (D / 4)) * 4;
@@ -458,10 +463,21 @@ __global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapPara
             state = ((uint64_t)task * p.num_q_heads + q_head) * p.max_q_tokens + token_offset;
         }
         if (mode == kMapPartialF32) {
-            *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.out) + state * D + d) = value;
+            float* target = reinterpret_cast<float*>(p.out) + state * D + d;
+            if (fused) {
+                coherent_store_u64(target, (uint64_t)__float_as_uint(value[0]) | ((uint64_t)__float_as_uint(value[1]) << 32));
+                coherent_store_u64(target + 2, (uint64_t)__float_as_uint(value[2]) | ((uint64_t)__float_as_uint(value[3]) << 32));
+            } else {
+                *reinterpret_cast<f32x4*>(target) = value;
+            }
         } else {
             const uint2 packed = make_uint2(pack_bf16x2(value[0], value[1]), pack_bf16x2(value[2], value[3]));
-            *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.out) + state * D + d) = packed;
+            uint16_t* target = reinterpret_cast<uint16_t*>(p.out) + state * D + d;
+            if (fused) {
+                coherent_store_u64(target, (uint64_t)packed.x | ((uint64_t)packed.y << 32));
+            } else {
+                *reinterpret_cast<uint2*>(target) = packed;
+            }
         }
     }
     if (mode != kMapDirectBf16 && tid < COLS) {
@@ -470,8 +486,80 @@ __global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapPara
         const uint32_t local_head = c - token_offset * p.max_q_heads;
         if (token_offset < num_q && local_head < num_heads) {
             const uint64_t state = ((uint64_t)task * p.num_q_heads + first_q_head + local_head) * p.max_q_tokens + token_offset;
-            p.max_logits[state] = stats_lds[(NWAVES * COLS + c) * 2];
-            p.exp_sums[state] = stats_lds[(NWAVES * COLS + c) * 2 + 1];
+            if (fused) {
+                coherent_store_f32(p.max_logits + state, stats_lds[(NWAVES * COLS + c) * 2]);
+                coherent_store_f32(p.exp_sums + state, stats_lds[(NWAVES * COLS + c) * 2 + 1]);
+            } else {
+                p.max_logits[state] = stats_lds[(NWAVES * COLS + c) * 2];
+                p.exp_sums[state] = stats_lds[(NWAVES * COLS + c) * 2 + 1];
+            }
+        }
+    }
+
+    // ---- fused Reduce: the last block of a (Q range, head group) merges all of its partial states ----------
+    if (!fused) return;
+    // The partial state above went out through device-coherent stores.  The barrier's release makes every
+    // wave wait for its stores to complete before thread 0 signals arrival; no L2 write-back is involved.
+    __syncthreads();
+    uint32_t* flag_lds = reinterpret_cast<uint32_t*>(stats_lds);
+    const uint32_t partial_begin = p.cu_partial_outputs[range_index];
+    uint32_t partial_end = p.cu_partial_outputs[range_index + 1];
+    if (partial_end > num_active_splits) partial_end = num_active_splits;
+    if (tid == 0) {
+        uint32_t* counter = p.arrival_counters + (uint64_t)range_index * gridDim.y + blockIdx.y;
+        const uint32_t arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+        const uint32_t last = arrived == partial_end - partial_begin ? 1u : 0u;
+        if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // re-arm for the next launch
+        flag_lds[0] = last;
+    }
+    __syncthreads();
+    if (flag_lds[0] == 0u) return;
+#ifdef KHM_EXPERIMENT_SKIP_MERGE
+    return;
+#endif
+    {
+        // Work units are (column, partial-slice) pairs; a group of D/4 lanes owns one unit at a time and walks
+        // its partials with an online merge, eight partials' loads in flight at once.  With at least as many
+        // columns as groups every column has one slice and a group writes its column's output directly;
+        // with fewer columns the spare groups split the partial list and combine through LDS.
+        constexpr int CHUNKS = D / 4;
+        constexpr int GROUPS = NWAVES * 64 / CHUNKS;
+        const int chunk = tid % CHUNKS;
+        const uint32_t group = tid / CHUNKS;
+        const uint32_t active_cols = num_q * p.max_q_heads;
+        const uint32_t slices = active_cols >= (uint32_t)GROUPS ? 1u : (uint32_t)GROUPS / active_cols;
+        const uint32_t num_units = active_cols * slices;
+        float* unit_acc = o_lds;                 // [GROUPS][D]
+        float* unit_stats = o_lds + GROUPS * D;  // [GROUPS][2]
+        const bool f32_partials = mode == kMapPartialF32;
+        for (uint32_t base = 0; base < num_units; base += GROUPS) {
+            const uint32_t unit = base + group;
+            const bool has_unit = unit < num_units;
+            const uint32_t c = has_unit ? unit / slices : 0u;
+            const uint32_t slice = unit - c * slices;
+            const uint32_t token_offset = c / p.max_q_heads;
+            const uint32_t local_head = c - token_offset * p.max_q_heads;
+            const bool live = has_unit && local_head < num_heads;
+            const uint32_t q_head = first_q_head + (live ? local_head : 0u);
+            MergeState state = merge_state_empty();
+            if (live) {
+                merge_partial_slice<D, true>(state, p.max_logits, p.exp_sums, p.out, f32_partials, partial_begin + slice, partial_end, slices,
+                                             partial_begin, p.num_q_heads, q_head, p.max_q_tokens, token_offset, chunk);
+            }
+            if (slices > 1u) {
+                if (chunk == 0) {
+                    unit_stats[group * 2] = state.run_max;
+                    unit_stats[group * 2 + 1] = state.run_sum;
+                }
+                *reinterpret_cast<f32x4*>(unit_acc + group * D + chunk * 4) = state.acc;
+                __syncthreads();
+                if (live && slice == 0u) state = merge_combine_slices<D>(unit_stats, unit_acc, group, slices, chunk);
+            }
+            if (live && slice == 0u) {
+                const uint64_t out_index = ((uint64_t)(flat_begin + token_offset) * p.num_q_heads + q_head) * D + chunk * 4;
+                merge_store_output(state, p.final_output, p.gates, out_index);
+            }
+            if (slices > 1u) __syncthreads();
         }
     }
 }

@@ -128,6 +128,26 @@ class Compute:
                                                 num_active_kv_splits, param_block(replay_parameters),
                                                 stream_handle(stream)))
 
+    def arrival_counters_bytes(self) -> int:
+        c, s = self.config.c(), self.shape.c()
+        return int(_lib.lib().khm_sliced_kv_arrival_counters_bytes(ctypes.byref(c), ctypes.byref(self.execution), ctypes.byref(s)))
+
+    def invoke_map_reduce(self, *, q, kv_pages, req_slots, page_ids, sdpa_map_task_templates, partial_exp_sums,
+                          partial_max_logits, partial_output, cu_sdpa_partial_outputs, output, arrival_counters,
+                          page_table_index: ReplayU32, num_active_tokens: ReplayU32, num_active_kv_splits: ReplayU32,
+                          gates=None, replay_parameters=None, stream=None) -> None:
+        """Map and Reduce (optionally gated) in one launch; `arrival_counters` must start zeroed."""
+        map_buffers = SlicedKvMapBuffers(view(q), view(kv_pages), view(req_slots), view(page_ids),
+                                         view(sdpa_map_task_templates), view(partial_exp_sums), view(partial_max_logits),
+                                         view(partial_output))
+        reduce_buffers = SlicedKvReduceBuffers(view(partial_exp_sums), view(partial_max_logits), view(partial_output),
+                                               view(cu_sdpa_partial_outputs), view(output))
+        gate_view = view(gates) if gates is not None else _lib.Buffer(None, 0)
+        _lib.check(_lib.lib().khm_sliced_kv_map_reduce(self._handle, ctypes.byref(map_buffers), ctypes.byref(reduce_buffers),
+                                                       gate_view, view(arrival_counters), page_table_index, num_active_tokens,
+                                                       num_active_kv_splits, param_block(replay_parameters),
+                                                       stream_handle(stream)))
+
     def invoke_reduce(self, *, partial_exp_sums, partial_max_logits, partial_output, cu_sdpa_partial_outputs, output,
                       num_active_tokens: ReplayU32, gates=None, replay_parameters=None, stream=None) -> None:
         buffers = SlicedKvReduceBuffers(view(partial_exp_sums), view(partial_max_logits), view(partial_output),

@@ -75,6 +75,26 @@ class Compute:
                                                num_active_q_token_tiles, num_active_kv_splits,
                                                param_block(replay_parameters), stream_handle(stream)))
 
+    def arrival_counters_bytes(self) -> int:
+        c, s = self.config.c(), self.shape.c()
+        return int(_lib.lib().khm_sliced_q_arrival_counters_bytes(ctypes.byref(c), ctypes.byref(self.execution), ctypes.byref(s)))
+
+    def invoke_map_reduce(self, *, q, kv_pages, req_slots, page_ids, visible_kv_token_ranges, q_token_ranges,
+                          sdpa_map_task_templates, partial_output, partial_exp_sums, partial_max_logits,
+                          cu_sdpa_partial_outputs, output, arrival_counters, page_table_index: ReplayU32,
+                          num_active_tokens: ReplayU32, num_active_q_token_tiles: ReplayU32, num_active_kv_splits: ReplayU32,
+                          replay_parameters=None, stream=None) -> None:
+        """Map and Reduce in one launch; `arrival_counters` must start zeroed."""
+        map_buffers = SlicedQMapBuffers(view(q), view(kv_pages), view(req_slots), view(page_ids),
+                                        view(visible_kv_token_ranges), view(q_token_ranges), view(sdpa_map_task_templates),
+                                        view(partial_output), view(partial_exp_sums), view(partial_max_logits))
+        reduce_buffers = SlicedQReduceBuffers(view(partial_output), view(partial_exp_sums), view(partial_max_logits),
+                                              view(q_token_ranges), view(cu_sdpa_partial_outputs), view(output))
+        _lib.check(_lib.lib().khm_sliced_q_map_reduce(self._handle, ctypes.byref(map_buffers), ctypes.byref(reduce_buffers),
+                                                      view(arrival_counters), page_table_index, num_active_tokens,
+                                                      num_active_q_token_tiles, num_active_kv_splits,
+                                                      param_block(replay_parameters), stream_handle(stream)))
+
     def invoke_direct(self, *, q, kv_pages, req_slots, page_ids, visible_kv_token_ranges, q_token_ranges,
                       sdpa_map_task_templates, output, page_table_index: ReplayU32, num_active_tokens: ReplayU32,
                       num_active_q_token_tiles: ReplayU32, replay_parameters=None, stream=None) -> None:
