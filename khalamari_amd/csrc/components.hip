@@ -9,6 +9,7 @@
 #include "device_params.h"
 #include "reduce_gate.hip.h"
 #include "split_kv_map.hip.h"
+#include "tile_map.hip.h"
 
 namespace khm {
 
@@ -37,6 +38,25 @@ static MapKernel select_small_tile_kernel(uint32_t head_dim, uint32_t column_til
         }
     }
     return nullptr;
+}
+
+struct TileKernelChoice {
+    MapKernel kernel;
+    uint32_t threads;
+    uint32_t smem_bytes;
+};
+
+// Tiled (LDS-shared K/V) kernel for Q tiles of 65..256 coordinates.
+static TileKernelChoice select_tile_kernel(uint32_t head_dim, uint32_t coordinates) {
+    if (head_dim == 128) {
+        if (coordinates <= 128) return {tile_map_kernel<128, 2, 4, 64>, 256, (uint32_t)TileSmem<128, 64>::kBytes};
+        return {tile_map_kernel<128, 4, 4, 64>, 256, (uint32_t)TileSmem<128, 64>::kBytes};
+    }
+    if (head_dim == 256) {
+        if (coordinates <= 128) return {tile_map_kernel<256, 2, 4, 32>, 256, (uint32_t)TileSmem<256, 32>::kBytes};
+        return {tile_map_kernel<256, 2, 8, 32>, 512, (uint32_t)TileSmem<256, 32>::kBytes};
+    }
+    return {nullptr, 0, 0};
 }
 
 static ReduceKernel select_reduce_kernel(uint32_t head_dim, bool ranged) {
@@ -119,6 +139,8 @@ struct ComputeBase {
     ReduceKernel reduce;
     uint32_t tokens_per_page;
     uint32_t num_q_head_ranges;
+    uint32_t map_threads;
+    uint32_t map_smem_bytes;
     bool direct;
 };
 
@@ -216,6 +238,8 @@ extern "C" int khm_sliced_kv_create(const khm_gqa_sdpa_config* config, const khm
     compute->num_q_head_ranges = div_ceil_u32(sdpa.num_q_heads / sdpa.num_kv_heads, variant->map_max_q_heads);
     compute->direct = false;
     compute->map = select_small_tile_kernel(config->head_dim, div_ceil_u32(variant->map_max_q_heads, 16));
+    compute->map_threads = kMapWaves * 64;
+    compute->map_smem_bytes = 0;
     compute->reduce = select_reduce_kernel(config->head_dim, false);
     if (compute->map == nullptr || compute->reduce == nullptr) {
         delete compute;
@@ -391,7 +415,8 @@ extern "C" int khm_sliced_q_create(const khm_gqa_sdpa_config* config, const khm_
     KHM_REQUIRE(!mul_overflows_u32(shape->num_total_sdpa_map_task_templates, 3),
                 "GQA SplitKV SlicedQ map TaskTemplate metadata exceeds the shader u32 element-index domain");
     std::string why;
-    if (kernel_family(sdpa, *variant, config->kv_dtype, &why) != 1) return fail(KHM_ERR_UNSUPPORTED, "%s", why.c_str());
+    const int family = kernel_family(sdpa, *variant, config->kv_dtype, &why);
+    if (family == 0) return fail(KHM_ERR_UNSUPPORTED, "%s", why.c_str());
     auto* compute = new khm_sliced_q();
     compute->config = *config;
     compute->variant = *variant;
@@ -399,7 +424,26 @@ extern "C" int khm_sliced_q_create(const khm_gqa_sdpa_config* config, const khm_
     compute->tokens_per_page = sdpa.tokens_per_page;
     compute->num_q_head_ranges = div_ceil_u32(sdpa.num_q_heads / sdpa.num_kv_heads, variant->map_max_q_heads);
     compute->direct = direct_output != 0;
-    compute->map = select_small_tile_kernel(config->head_dim, div_ceil_u32(variant->map_max_q_tokens * variant->map_max_q_heads, 16));
+    const uint32_t coordinates = variant->map_max_q_tokens * variant->map_max_q_heads;
+    if (family == 1) {
+        compute->map = select_small_tile_kernel(config->head_dim, div_ceil_u32(coordinates, 16));
+        compute->map_threads = kMapWaves * 64;
+        compute->map_smem_bytes = 0;
+    } else {
+        const TileKernelChoice choice = select_tile_kernel(config->head_dim, coordinates);
+        compute->map = choice.kernel;
+        compute->map_threads = choice.threads;
+        compute->map_smem_bytes = choice.smem_bytes;
+        if (choice.kernel != nullptr) {
+            // more than 64 KB of LDS per block has to be requested once per kernel
+            const hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void*>(choice.kernel),
+                                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)choice.smem_bytes);
+            if (status != hipSuccess) {
+                delete compute;
+                return fail(KHM_ERR_HIP, "could not reserve %u bytes of LDS: %s", choice.smem_bytes, hipGetErrorString(status));
+            }
+        }
+    }
     compute->reduce = select_reduce_kernel(config->head_dim, true);
     if (compute->map == nullptr || compute->reduce == nullptr) {
         delete compute;
@@ -467,7 +511,7 @@ static int launch_sliced_q_map(const khm_sliced_q* compute, const khm_buffer& q,
         p.gates = fused->gates;
     }
     const dim3 grid(shape.num_total_sdpa_map_task_templates, config.num_kv_heads * compute->num_q_head_ranges, 1);
-    hipLaunchKernelGGL(compute->map, grid, dim3(kMapWaves * 64), 0, static_cast<hipStream_t>(stream), p);
+    hipLaunchKernelGGL(compute->map, grid, dim3(compute->map_threads), compute->map_smem_bytes, static_cast<hipStream_t>(stream), p);
     return check_launch("sliced-Q map");
 }
 

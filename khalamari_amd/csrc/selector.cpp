@@ -279,7 +279,8 @@ static int validate_request_shapes(const khm_selector& selector, const khm_reque
 //       q == 1           -> SlicedKv with all of a KV head's Q heads in one block when ratio <= 8,
 //                           otherwise a one-token sliced-Q tile that still reads K/V once per KV head.
 //       q * ratio <= 64  -> one sliced-Q tile of q tokens x ratio heads (verify blocks).
-//       larger           -> the largest power-of-two token tile with tile * ratio <= 64.
+//       q >= 16          -> dense prefill: the largest power-of-two token tile with tile * ratio <= 256.
+//       otherwise        -> the largest power-of-two token tile with tile * ratio <= 64.
 //   * KV slice.  A block streams its slice once, so slices only need to be short enough to fill the
 //     chip: aim for kTargetBlocks blocks in total, never below kMinSlice tokens (shorter slices pay
 //     more in partial traffic than they gain in parallelism), never above the longest context.
@@ -287,7 +288,8 @@ static int validate_request_shapes(const khm_selector& selector, const khm_reque
 // ---------------------------------------------------------------------------------------------
 constexpr uint64_t kTargetBlocks = 1024;
 constexpr uint32_t kMinSlice = 256;
-constexpr uint32_t kMaxColumns = 64;
+constexpr uint32_t kMaxColumns = 64;          // small-tile split-KV kernel (decode, verify)
+constexpr uint32_t kMaxPrefillColumns = 256;  // LDS-shared K/V tile kernel (dense prefill chunks)
 
 static int lookup_variant(const khm_sdpa_config& config, uint32_t queries, khm_sdpa_variant* out) {
     const uint32_t ratio = ratio_of(config);
@@ -295,9 +297,12 @@ static int lookup_variant(const khm_sdpa_config& config, uint32_t queries, khm_s
         const uint32_t clamped = std::min(std::max(config.head_dim, 32u), 256u);
         return khm_sdpa_variant_sliced_kv(&config, next_power_of_two(clamped), 128, ratio, out);
     }
-    uint32_t heads = std::min(ratio, kMaxColumns);
+    // Chunks of 16+ tokens per request are compute-bound: give them the widest tile so each K/V byte staged in
+    // LDS feeds as many MFMA columns as possible.  Narrower blocks are bandwidth-bound and stay on small tiles.
+    const uint32_t max_columns = queries >= 16 ? kMaxPrefillColumns : kMaxColumns;
+    uint32_t heads = std::min(ratio, max_columns);
     uint32_t tile = queries;
-    while (tile > 1 && (uint64_t)tile * heads > kMaxColumns) tile /= 2;
+    while (tile > 1 && (uint64_t)tile * heads > max_columns) tile /= 2;
     return khm_sdpa_variant_sliced_q(&config, KHM_MAP_Q_TOKENS_AND_HEADS, tile, 64, heads, out);
 }
 

@@ -293,7 +293,9 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
             }
         }
         const bool interior = first_token >= all_lo && first_token + 16 <= all_hi;
-        uint32_t p_bits[NT][2];
+        // Softmax weights go into the second MFMA as hi + lo bf16 pairs (p = hi + lo to ~2^-17): this kernel is
+        // bandwidth-bound, so the second product is free and the weights keep f32-like accuracy as in the reference.
+        uint32_t p_bits[NT][2], p_low[NT][2];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             float v[4];
@@ -319,6 +321,8 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
             run_sum[nt] = run_sum[nt] * alpha + ((e[0] + e[1]) + (e[2] + e[3]));
             p_bits[nt][0] = pack_bf16x2(e[0], e[1]);
             p_bits[nt][1] = pack_bf16x2(e[2], e[3]);
+            p_low[nt][0] = pack_bf16x2(e[0] - bf16_bits_to_f32(p_bits[nt][0] & 0xffffu), e[1] - bf16_bits_to_f32(p_bits[nt][0] >> 16));
+            p_low[nt][1] = pack_bf16x2(e[2] - bf16_bits_to_f32(p_bits[nt][1] & 0xffffu), e[3] - bf16_bits_to_f32(p_bits[nt][1] >> 16));
             if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) acc[nt][mt] *= alpha;
@@ -358,7 +362,9 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const uint2 b_bits = make_uint2(p_bits[nt][0], p_bits[nt][1]);
+                const uint2 b_low = make_uint2(p_low[nt][0], p_low[nt][1]);
                 acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, __builtin_bit_cast(s16x4, b_bits), acc[nt][mt], 0, 0, 0);
+                acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, __builtin_bit_cast(s16x4, b_low), acc[nt][mt], 0, 0, 0);
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

@@ -102,6 +102,10 @@ def test_replay_paged_ranges(device, head_dim, tpp):
     (sdpa.MAP_Q_TOKENS_PER_HEAD, 12, 1, 6, 64, 128),
     (sdpa.MAP_Q_TOKENS_PER_HEAD, 6, 32, 1, 8, 128),
     (sdpa.MAP_Q_HEADS_PER_TOKEN, 5, 4, 3, 64, 256),
+    (sdpa.MAP_Q_HEADS_PER_TOKEN, 8, 32, 8, 128, 256),
+    (sdpa.MAP_Q_TOKENS_AND_HEADS, 12, 16, 12, 64, 256),
+    (sdpa.MAP_Q_TOKENS_AND_HEADS, 8, 16, 8, 64, 128),
+    (sdpa.MAP_Q_TOKENS_AND_HEADS, 8, 32, 8, 64, 128),
 ])
 def test_q_token_head_assignments_and_direct_output(device, kind, ratio, tile, heads, stage, head_dim):
     """sliced_q_test.rs:219-401: tile/head geometries x {split, direct}, reversed pages, windowed and empty ranges."""
@@ -326,3 +330,21 @@ def test_selector_and_metadata_drive_the_kernels_end_to_end(device):
         actual = gpu_runner.bf16_tensor_to_f32(out)
         helpers.assert_parity(actual[:w.num_tokens], helpers.expected_output(w), f"end-to-end {histories} {q_lens}")
         assert np.all(out[w.num_tokens:].cpu().numpy() == POISON)
+
+
+@pytest.mark.parametrize("hq,hkv,d,tile", [(64, 8, 128, 32), (32, 4, 128, 16), (24, 4, 256, 16), (16, 2, 256, 32)])
+def test_chunked_prefill_onto_a_paged_prefix(device, hq, hkv, d, tile):
+    """Config-5 shape at reduced size: causal chunks appended to paged prefixes (including an empty prefix), wide
+    Q tiles on the LDS-shared K/V kernel, direct output and split-KV + Reduce."""
+    histories = [0, 333, 1000]
+    q_lens = [150, 64, 37]
+    w = helpers.make_workload(num_q_heads=hq, num_kv_heads=hkv, head_dim=d, tokens_per_page=16, histories=histories,
+                              q_lens=q_lens, seed=90 + tile, garbage_bits=0x7FC0)
+    expected = helpers.expected_output(w)
+    ratio = hq // hkv
+    for kv_slice, direct in [(1 << 20, True), (256, False), (100, False)]:
+        ranges, templates, cu = helpers.fixed_slice_plan(histories, q_lens, tile, kv_slice)
+        print(f"prefill hq={hq} hkv={hkv} d={d} tile={tile} kv_slice={kv_slice} direct={direct}", flush=True)
+        actual = gpu_runner.run_sliced_q(w, ranges, templates, cu, device, kind=sdpa.MAP_Q_TOKENS_AND_HEADS, max_q_tokens=tile,
+                                         max_q_heads=ratio, stage=64, direct=direct)
+        helpers.assert_parity(actual, expected, f"prefill tile={tile} slice={kv_slice} direct={direct}")
