@@ -49,12 +49,16 @@ struct TileKernelChoice {
 // Tiled (LDS-shared K/V) kernel for Q tiles of 65..256 coordinates.
 static TileKernelChoice select_tile_kernel(uint32_t head_dim, uint32_t coordinates) {
     if (head_dim == 128) {
-        if (coordinates <= 128) return {tile_map_kernel<128, 2, 4, 64>, 256, (uint32_t)TileSmem<128, 64>::kBytes};
-        return {tile_map_kernel<128, 4, 4, 64>, 256, (uint32_t)TileSmem<128, 64>::kBytes};
+        if (coordinates <= 128) return {tile_map_kernel<128, 2, 4, 64, 4, 2>, 256, (uint32_t)TileSmem<128, 64, 4>::kBytes};
+#ifdef KHM_X_TILE_B
+        return {tile_map_kernel<128, 4, 4, 64, 4, 1>, 256, (uint32_t)TileSmem<128, 64, 4>::kBytes};
+#else
+        return {tile_map_kernel<128, 2, 8, 64, 4, 1>, 512, (uint32_t)TileSmem<128, 64, 4>::kBytes};
+#endif
     }
     if (head_dim == 256) {
-        if (coordinates <= 128) return {tile_map_kernel<256, 2, 4, 32>, 256, (uint32_t)TileSmem<256, 32>::kBytes};
-        return {tile_map_kernel<256, 2, 8, 32>, 512, (uint32_t)TileSmem<256, 32>::kBytes};
+        if (coordinates <= 128) return {tile_map_kernel<256, 2, 4, 32, 4, 1>, 256, (uint32_t)TileSmem<256, 32, 4>::kBytes};
+        return {tile_map_kernel<256, 2, 8, 32, 4, 1>, 512, (uint32_t)TileSmem<256, 32, 4>::kBytes};
     }
     return {nullptr, 0, 0};
 }

@@ -7,31 +7,38 @@
 //
 // Work shape.  A block owns up to NWAVES * NTW * 16 (q_token, q_head) columns; each wave owns NTW 16-column
 // tiles for the whole KV range, so there is no cross-wave merge.  KV is walked in BK-token tiles that all
-// waves share through LDS.  Per tile and wave:
-//     S^T[BK][cols] = K . Q^T        v_mfma_f32_16x16x32_bf16, K rows (ds_read_b128) as the A operand, Q in registers
-//     online softmax per column      exp2 domain; the accumulator is rescaled only when a column's maximum moved
+// waves share through LDS, 32 tokens (one "slice") at a time:
+//     S^T[32][cols] = K . Q^T        v_mfma_f32_16x16x32_bf16, K rows (ds_read_b128) as the A operand, Q in registers
+//     online softmax per column      exp2 domain; the accumulator is rescaled only when a column's maximum moved far
 //     O^T[D][cols] += V^T . P^T      v_mfma_f32_16x16x32_bf16; the V^T operand comes from row-major V in LDS through
 //                                    ds_read_b64_tr_b16 (each lane receives 4 tokens of one dim), P stays in registers
-// Memory.  The block loads tile i+2 from HBM (fully coalesced 16-byte chunks, one 16-token page slab per pass)
-// into registers while it computes tile i; LDS is double-buffered so one barrier per tile suffices.
+// Memory.  K/V tiles go from HBM/L2 straight into LDS (global_load_lds_dwordx4, 1 KB per wave instruction) without
+// passing through registers; NSTAGES tiles are in flight and one barrier per tile publishes them.  A direct load
+// writes 64 consecutive 16-byte chunks, so rows cannot be padded; instead each lane fetches the chunk whose index is
+// XOR-swizzled with the row, which makes both the b128 K reads and the transposed V reads bank-conflict free.
 // Blocks are renumbered so that each XCD walks a contiguous run of the (KV head, template) list: the Q ranges of
 // one sequence share their K/V through that XCD's L2 instead of each pulling it from HBM.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "device_math.hip.h"
 #include "device_params.h"
 
+#ifndef KHM_X_PRECISE
+#define KHM_X_PRECISE true
+#endif
 namespace khm {
 
 typedef short s16x4v __attribute__((ext_vector_type(4)));
 
-template <int D, int BK>
+template <int D, int BK, int NSTAGES>
 struct TileSmem {
-    static constexpr int kRowBytes = D * 2 + 32;   // 32 B pad: conflict-light b128 and transposed reads
+    static constexpr int kRowBytes = D * 2;
     static constexpr int kTileBytes = BK * kRowBytes;
-    static constexpr int kBytes = 2 /*K,V*/ * 2 /*stages*/ * kTileBytes;
+    static constexpr int kBytes = 2 /*K,V*/ * NSTAGES * kTileBytes;
 };
 
 // LDS transpose read: lane r of every 16-lane group passes the address of 4 consecutive bf16; lane i receives
@@ -40,22 +47,37 @@ __device__ __forceinline__ s16x4v lds_read_tr16(const unsigned char* address) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4v __attribute__((address_space(3)))*)(address));
 }
 
-template <int D, int NTW, int NWAVES, int BK>
-__global__ __launch_bounds__(NWAVES * 64) void tile_map_kernel(const MapParams p) {
-    constexpr int THREADS = NWAVES * 64;
+// 16 bytes per lane from global memory to LDS: lane l of the wave lands at lds_base + 16 * l (lds_base is wave-uniform).
+__device__ __forceinline__ void load_to_lds_b128(const unsigned char* source, unsigned char* lds_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)source,
+                                     (__attribute__((address_space(3))) void*)lds_base, 16, 0, 0);
+}
+
+// Wait until at most COUNT of this wave's vector-memory operations are still in flight (they retire in order).
+template <int COUNT>
+__device__ __forceinline__ void wait_vmem_outstanding() {
+    static_assert(COUNT >= 0 && COUNT < 64, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(COUNT) : "memory");
+}
+
+template <int D, int NTW, int NWAVES, int BK, int NSTAGES, int MIN_BLOCKS>
+__global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const MapParams p) {
     constexpr int KS = D / 32;                      // QK k-steps
     constexpr int MT = D / 16;                      // PV dim tiles
-    constexpr int RT = BK / 16;                     // 16-token row tiles per KV tile
-    constexpr int CHUNKS_PER_ROW = D / 8;           // 16-byte chunks per K/V row
-    constexpr int ROWS_PER_PASS = THREADS / CHUNKS_PER_ROW;
-    constexpr int PASSES = BK / ROWS_PER_PASS;      // global->LDS passes per plane
-    static_assert(ROWS_PER_PASS <= 16 && 16 % ROWS_PER_PASS == 0, "a load pass must stay inside one 16-token group");
-    static_assert(BK % 32 == 0, "PV consumes 32 tokens per MFMA");
-    using Smem = TileSmem<D, BK>;
+    constexpr int SL = BK / 32;                     // slices per tile
+    constexpr int CPR = D / 8;                      // 16-byte chunks per K/V row
+    constexpr int RPL = 64 / CPR;                   // rows per wave load
+    constexpr int UNITS = BK / RPL;                 // wave loads per plane and tile
+    constexpr int UPW = UNITS / NWAVES;             // ... per wave
+    constexpr int LPW = 2 * UPW;                    // K + V loads per wave and tile
+    static_assert(UNITS % NWAVES == 0 && UPW >= 1, "tile loads must divide evenly over the waves");
+    static_assert((SL == 1 || SL == 2) && NSTAGES >= 3 && NSTAGES <= 5, "unsupported tiling");
+    using Smem = TileSmem<D, BK, NSTAGES>;
+    constexpr int ROW = Smem::kRowBytes;
 
-    extern __shared__ __align__(16) unsigned char tile_smem[];
-    unsigned char* k_lds = tile_smem;                              // [2][BK][kRowBytes]
-    unsigned char* v_lds = tile_smem + 2 * Smem::kTileBytes;       // [2][BK][kRowBytes]
+    extern __shared__ __align__(1024) unsigned char tile_smem[];
+    unsigned char* k_lds = tile_smem;                                    // [NSTAGES][BK][ROW]
+    unsigned char* v_lds = tile_smem + NSTAGES * Smem::kTileBytes;       // [NSTAGES][BK][ROW]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -102,7 +124,9 @@ __global__ __launch_bounds__(NWAVES * 64) void tile_map_kernel(const MapParams p
     const uint32_t first_q_head = kv_head * p.q_heads_per_kv_head + head_range_begin;
 
     // ---- per-lane column facts ---------------------------------------------------------------------------
-    uint32_t col_lo[NTW], col_hi[NTW], col_token[NTW], col_head[NTW];
+    auto column_token = [&](int nt) { return (uint32_t)((wave * NTW + nt) * 16 + r16) / p.max_q_heads; };
+    auto column_head = [&](int nt) { return (uint32_t)((wave * NTW + nt) * 16 + r16) % p.max_q_heads; };
+    uint32_t col_lo[NTW], col_hi[NTW];
     bool col_active[NTW];
     uint32_t blk_lo = 0xffffffffu, blk_hi = 0u, wave_all_lo = 0u, wave_all_hi = 0xffffffffu, min_span = 0xffffffffu;
 #pragma unroll
@@ -111,8 +135,6 @@ __global__ __launch_bounds__(NWAVES * 64) void tile_map_kernel(const MapParams p
         const uint32_t token_offset = c / p.max_q_heads;
         const uint32_t local_head = c - token_offset * p.max_q_heads;
         col_active[nt] = token_offset < num_q && local_head < num_heads;
-        col_token[nt] = token_offset;
-        col_head[nt] = local_head;
         uint32_t lo = kv_begin, hi = kv_end;
         if (col_active[nt]) {
             const uint64_t token = flat_begin + token_offset;
@@ -124,6 +146,7 @@ __global__ __launch_bounds__(NWAVES * 64) void tile_map_kernel(const MapParams p
         if (hi < lo) hi = lo;
         col_lo[nt] = lo;
         col_hi[nt] = hi;
+        // padding columns carry a zero Q row and are never stored, so they do not constrain anything
         if (col_active[nt]) {
             if (hi > lo) {
                 blk_lo = lo < blk_lo ? lo : blk_lo;
@@ -143,33 +166,36 @@ __global__ __launch_bounds__(NWAVES * 64) void tile_map_kernel(const MapParams p
         other = __shfl_xor(wave_all_hi, offset); wave_all_hi = other < wave_all_hi ? other : wave_all_hi;
         other = __shfl_xor(min_span, offset); min_span = other < min_span ? other : min_span;
     }
-    // Rounding a softmax weight to bf16 costs up to 2^-9 of that weight; with few keys the weights are O(1) and
-    // the error shows at the 1e-3 level.  Waves whose columns see at most kPreciseSpan keys therefore feed the second
-    // MFMA with hi + lo bf16 pairs (the reference keeps P in f32); long contexts, where every weight is small, use one.
-    constexpr uint32_t kPreciseSpan = 256;
-    const bool precise = __builtin_amdgcn_readfirstlane(min_span) <= kPreciseSpan;
+    // a slice is "interior" for the wave when every active column of the wave sees all of its 32 tokens
     wave_all_lo = __builtin_amdgcn_readfirstlane(wave_all_lo);
     wave_all_hi = __builtin_amdgcn_readfirstlane(wave_all_hi);
-    // block-wide KV range: reduce the per-wave ranges through LDS
+    // block-wide KV range and shortest span: reduce the per-wave values through LDS
     uint32_t* range_lds = reinterpret_cast<uint32_t*>(tile_smem);
     if (lane == 0) {
-        range_lds[wave * 2] = blk_lo;
-        range_lds[wave * 2 + 1] = blk_hi;
+        range_lds[wave * 3] = blk_lo;
+        range_lds[wave * 3 + 1] = blk_hi;
+        range_lds[wave * 3 + 2] = min_span;
     }
     __syncthreads();
-    const uint32_t wave_lo = __builtin_amdgcn_readfirstlane(blk_lo);
-    const uint32_t wave_hi = __builtin_amdgcn_readfirstlane(blk_hi);
     blk_lo = 0xffffffffu;
     blk_hi = 0u;
+    min_span = 0xffffffffu;
 #pragma unroll
     for (int w = 0; w < NWAVES; ++w) {
-        const uint32_t lo = range_lds[w * 2], hi = range_lds[w * 2 + 1];
+        const uint32_t lo = range_lds[w * 3], hi = range_lds[w * 3 + 1], span = range_lds[w * 3 + 2];
         blk_lo = lo < blk_lo ? lo : blk_lo;
         blk_hi = hi > blk_hi ? hi : blk_hi;
+        min_span = span < min_span ? span : min_span;
     }
     blk_lo = __builtin_amdgcn_readfirstlane(blk_lo);
     blk_hi = __builtin_amdgcn_readfirstlane(blk_hi);
-    __syncthreads();
+    // Rounding a softmax weight to bf16 costs up to 2^-9 of that weight; with few keys the weights are O(1) and
+    // the error shows at the 1e-3 level.  Blocks with a column that sees at most kPreciseSpan keys therefore feed the
+    // second MFMA with hi + lo bf16 pairs (the reference keeps P in f32); long contexts, where every weight is small,
+    // use one.
+    constexpr uint32_t kPreciseSpan = 256;
+    const bool precise = KHM_X_PRECISE && (uint32_t)__builtin_amdgcn_readfirstlane(min_span) <= kPreciseSpan;
+    __syncthreads();   // range_lds is about to be overwritten by the first tile
     {
         const uint64_t table_tokens = (uint64_t)p.pages_per_request_layer << p.tokens_per_page_shift;
         if (blk_hi > table_tokens) blk_hi = (uint32_t)table_tokens;
@@ -182,7 +208,7 @@ __global__ __launch_bounds__(NWAVES * 64) void tile_map_kernel(const MapParams p
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) q_frag[nt][ks] = make_uint4(0, 0, 0, 0);
         if (col_active[nt]) {
-            const uint16_t* row = p.q + ((uint64_t)(flat_begin + col_token[nt]) * p.num_q_heads + first_q_head + col_head[nt]) * D;
+            const uint16_t* row = p.q + ((uint64_t)(flat_begin + column_token(nt)) * p.num_q_heads + first_q_head + column_head(nt)) * D;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) q_frag[nt][ks] = *reinterpret_cast<const uint4*>(row + ks * 32 + g * 8);
         }
@@ -191,197 +217,226 @@ __global__ __launch_bounds__(NWAVES * 64) void tile_map_kernel(const MapParams p
     // ---- tile schedule -------------------------------------------------------------------------------------
     const uint32_t first_group = blk_lo >> 4;                                   // 16-token groups
     const uint32_t num_groups = blk_hi > blk_lo ? ((blk_hi - 1) >> 4) - first_group + 1 : 0;
-    const uint32_t num_tiles = (num_groups + RT - 1) / RT;
+    const uint32_t num_slices = (num_groups + 1) / 2;
+    const uint32_t num_tiles = (num_slices + SL - 1) / SL;
+    const uint32_t first_token = first_group << 4;
     const uint32_t* table = p.page_ids + ((uint64_t)req_slot * p.num_gqa_layers + layer) * p.pages_per_request_layer;
     const uint32_t tpp = p.tokens_per_page;
     const uint32_t tpp_shift = p.tokens_per_page_shift;
-    const uint64_t plane_k = ((uint64_t)kv_head * tpp) * (D * 2);
-    const uint64_t plane_v = ((uint64_t)(p.num_kv_heads + kv_head) * tpp) * (D * 2);
+    const uint64_t plane_k = ((uint64_t)kv_head * tpp) * ROW;
+    const uint64_t plane_v = ((uint64_t)(p.num_kv_heads + kv_head) * tpp) * ROW;
 
-    // Page ids of 64 consecutive 16-token groups per register pair; two pairs alternate.
-    uint32_t ids_a[2] = {0, 0}, ids_b[2] = {0, 0};
-    auto load_ids = [&](uint32_t chunk, uint32_t (&ids)[2]) {
-        const uint32_t group = chunk * 64 + lane;
-        if (group < num_groups) {
-            const uint32_t token = (first_group + group) << 4;
-            const uint32_t last_page = p.pages_per_request_layer - 1;
-            const uint32_t page0 = token >> tpp_shift;
-            const uint32_t page1 = (token + 8) >> tpp_shift;
-            ids[0] = table[page0 < last_page ? page0 : last_page];
-            ids[1] = table[page1 < last_page ? page1 : last_page];
+    // A wave load covers RPL rows that lie inside one 8-token half of a 16-token group, before and after the clamp
+    // below, so its page is wave-uniform: the page id travels through a scalar load, fetched one iteration before the
+    // tile is issued, and the load address is a scalar base plus a 32-bit lane offset.
+    // Rows outside [blk_lo, blk_hi) may hold anything (unused page slots): their loads are redirected to the nearest
+    // visible token, so LDS only ever holds finite K/V and a zero weight really contributes zero.
+    typedef uint32_t TileIds __attribute__((ext_vector_type(UPW < 2 ? 2 : UPW)));
+    auto fetch_ids = [&](uint32_t tile) __attribute__((always_inline)) -> TileIds {
+        TileIds ids;
+        const uint32_t last_page = p.pages_per_request_layer - 1;
+#pragma unroll
+        for (int i = 0; i < UPW; ++i) {
+            uint32_t token = first_token + tile * BK + (wave * UPW + i) * RPL;
+            token = token < blk_lo ? blk_lo : token;
+            token = token >= blk_hi ? blk_hi - 1 : token;
+            const uint32_t page = token >> tpp_shift;
+            ids[i] = __builtin_amdgcn_readfirstlane(table[page < last_page ? page : last_page]);
+        }
+        return ids;
+    };
+    auto issue_tile = [&](uint32_t tile, const TileIds ids) __attribute__((always_inline)) {
+        const uint32_t stage = tile % NSTAGES;
+        // The lane-dependent address parts are a handful of VALU operations; the empty asm keeps the compiler from
+        // hoisting them out of the tile loop, where they would cost registers the accumulators need.
+        uint32_t lane_now = lane;
+        asm volatile("" : "+v"(lane_now));
+        const uint32_t load_row = lane_now / CPR;       // row inside a wave load
+        const uint32_t load_pos = lane_now % CPR;       // 16-byte position inside the row
+#pragma unroll
+        for (int i = 0; i < UPW; ++i) {
+            const uint32_t unit = wave * UPW + i;                                  // wave-uniform
+            const uint32_t row = unit * RPL + load_row;                            // row inside the tile
+            uint32_t token = first_token + tile * BK + row;
+            token = token < blk_lo ? blk_lo : token;
+            token = token >= blk_hi ? blk_hi - 1 : token;
+            const unsigned char* page = p.kv_pages + (uint64_t)ids[i] * p.page_bytes;   // scalar
+            const uint32_t in_page = (token & (tpp - 1)) * ROW;
+            const uint32_t k_offset_bytes = in_page + ((load_pos ^ (row & 15)) << 4);
+            const uint32_t v_offset_bytes = in_page + ((load_pos ^ ((row & 7) << 1)) << 4);
+            load_to_lds_b128(page + plane_k + k_offset_bytes, k_lds + stage * Smem::kTileBytes + unit * 1024);
+            load_to_lds_b128(page + plane_v + v_offset_bytes, v_lds + stage * Smem::kTileBytes + unit * 1024);
         }
     };
-    load_ids(0, ids_a);
-    if (num_groups > 64) load_ids(1, ids_b);
 
-    uint4 stage_k[PASSES], stage_v[PASSES];
-    const uint32_t load_row = tid / CHUNKS_PER_ROW;    // row inside a pass
-    const uint32_t load_chunk = tid % CHUNKS_PER_ROW;
-    auto load_tile = [&](uint32_t tile) {
+    // ---- LDS read addresses (per lane, relative to the slice) -------------------------------------------------------
+    // K: lane (r16, g) reads row rt*16 + r16, source chunk ks*4 + g, stored at position chunk ^ r16.
+    uint32_t k_offset[KS];
 #pragma unroll
-        for (int pass = 0; pass < PASSES; ++pass) {
-            const uint32_t row = pass * ROWS_PER_PASS + load_row;                // row inside the tile
-            uint32_t group = tile * RT + (row >> 4);
-            if (group >= num_groups) group = num_groups - 1;                     // tail rows: any valid page, masked below
-            const uint32_t chunk = group >> 6;
-            const uint32_t sel0 = (chunk & 1) ? ids_b[0] : ids_a[0];
-            const uint32_t sel1 = (chunk & 1) ? ids_b[1] : ids_a[1];
-            uint32_t id0 = __builtin_amdgcn_readlane(sel0, group & 63);
-            uint32_t id1 = __builtin_amdgcn_readlane(sel1, group & 63);
-            const uint32_t first_token = (first_group + group) << 4;
-            if (tpp == 8) {
-                if (first_token + 8 >= blk_hi) id1 = id0;
-                if (first_token + 8 <= blk_lo) id0 = id1;
-            }
-            const uint32_t row16 = row & 15;
-            const uint32_t in_page = (first_token + row16) & (tpp - 1);
-            const uint64_t page = row16 >= 8 ? id1 : id0;
-            const unsigned char* base = p.kv_pages + page * p.page_bytes + (uint64_t)in_page * (D * 2) + load_chunk * 16;
-            stage_k[pass] = *reinterpret_cast<const uint4*>(base + plane_k);
-            stage_v[pass] = *reinterpret_cast<const uint4*>(base + plane_v);
-        }
-    };
-    auto refresh_ids = [&](uint32_t tile) {
-        // Called once per tile by every wave (uniform): when the tile starts a new 64-group id chunk, prefetch the next one.
-        const uint32_t group = tile * RT;
-        const uint32_t chunk = group >> 6;
-        if ((group & 63) < (uint32_t)RT && chunk >= 1 && (chunk + 1) * 64 < num_groups) {
-            if ((chunk + 1) & 1) load_ids(chunk + 1, ids_b); else load_ids(chunk + 1, ids_a);
-        }
-    };
-    auto store_tile = [&](uint32_t tile, int stage) {
-        unsigned char* k_dst = k_lds + stage * Smem::kTileBytes;
-        unsigned char* v_dst = v_lds + stage * Smem::kTileBytes;
-#pragma unroll
-        for (int pass = 0; pass < PASSES; ++pass) {
-            const uint32_t row = pass * ROWS_PER_PASS + load_row;
-            const uint32_t token = ((first_group + tile * RT) << 4) + row;
-            uint4 v = stage_v[pass];
-            if (token < blk_lo || token >= blk_hi) v = make_uint4(0, 0, 0, 0);  // unused page slots may hold anything
-            *reinterpret_cast<uint4*>(k_dst + row * Smem::kRowBytes + load_chunk * 16) = stage_k[pass];
-            *reinterpret_cast<uint4*>(v_dst + row * Smem::kRowBytes + load_chunk * 16) = v;
-        }
-    };
+    for (int ks = 0; ks < KS; ++ks) k_offset[ks] = r16 * ROW + (((ks * 4 + g) ^ r16) << 4);
+    // V: lane (g, r) passes row 4g + r/4 (+16 for the second half), dims mt*16 + 4*(r%4) .. +3, i.e. source chunk
+    // 2*mt + (r%4)/2, stored at position chunk ^ 2*(row & 7).
+    const uint32_t v_row = g * 4 + (r16 >> 2);
+    const uint32_t v_swizzle = ((r16 & 3) >> 1) ^ ((v_row & 7) << 1);
+    const uint32_t v_base = v_row * ROW + (r16 & 1) * 8;
 
     // ---- online-softmax state ------------------------------------------------------------------------------
+    // ref_max is the exponent reference of a column (log2 domain); it only moves when the column's maximum has
+    // grown by more than kRescaleThreshold, so the accumulators are rescaled rarely.  top_max tracks the true maximum
+    // for the partial-state ABI; the stored exp-sum is restated against it in the epilogue.
+    constexpr float kRescaleThreshold = 8.0f;
     f32x4 acc[NTW][MT];
-    float run_max[NTW], run_sum[NTW];
+    float run_sum[NTW];
+    float ref_max[NTW], top_max[NTW];
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt) {
-        run_max[nt] = -INFINITY;
+        ref_max[nt] = -INFINITY;
+        top_max[nt] = -INFINITY;
         run_sum[nt] = 0.0f;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     }
 
-    auto compute_tile = [&](uint32_t tile, int stage) {
-        const uint32_t tile_first = (first_group + tile * RT) << 4;
-        // Tiles entirely outside this wave's own columns' ranges contribute nothing (causal skew inside the block).
-        if (tile_first >= wave_hi || tile_first + BK <= wave_lo) return;
-        const unsigned char* k_src = k_lds + stage * Smem::kTileBytes;
-        const unsigned char* v_src = v_lds + stage * Smem::kTileBytes;
-        f32x4 s[RT][NTW];
+    struct Scores {
+        f32x4 s[2][NTW];
+    };
+    // S^T of one 32-token slice
+    auto scores_of = [&](const unsigned char* k_src, Scores& out) __attribute__((always_inline)) {
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
+        for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-            for (int nt = 0; nt < NTW; ++nt) s[rt][nt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            for (int nt = 0; nt < NTW; ++nt) out.s[rt][nt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
-            for (int rt = 0; rt < RT; ++rt) {
-                const uint4 a_bits = *reinterpret_cast<const uint4*>(k_src + (rt * 16 + r16) * Smem::kRowBytes + (ks * 32 + g * 8) * 2);
-                const bf16x8 a = __builtin_bit_cast(bf16x8, a_bits);
+            for (int rt = 0; rt < 2; ++rt) {
+                const uint4 bits = *reinterpret_cast<const uint4*>(k_src + k_offset[ks] + rt * 16 * ROW);
+                const bf16x8 a = __builtin_bit_cast(bf16x8, bits);
 #pragma unroll
                 for (int nt = 0; nt < NTW; ++nt)
-                    s[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, q_frag[nt][ks]), s[rt][nt], 0, 0, 0);
-            }
-        }
-        const bool interior = tile_first >= wave_all_lo && tile_first + BK <= wave_all_hi;
-        uint32_t p_bits[RT][NTW][2], p_low[RT][NTW][2];
-#pragma unroll
-        for (int nt = 0; nt < NTW; ++nt) {
-            float tile_max = -INFINITY;
-#pragma unroll
-            for (int rt = 0; rt < RT; ++rt) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    float v = s[rt][nt][i];
-                    if (!interior) {
-                        const uint32_t token = tile_first + rt * 16 + g * 4 + i;
-                        v = (token >= col_lo[nt] && token < col_hi[nt]) ? v : -INFINITY;
-                        s[rt][nt][i] = v;
-                    }
-                    tile_max = fmaxf(tile_max, v);
-                }
-            }
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16));
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
-            tile_max *= p.scale_log2e;                                 // scale > 0: max commutes with the scaling
-            const float next_max = fmaxf(run_max[nt], tile_max);
-            const float safe_max = next_max == -INFINITY ? 0.0f : next_max;
-            const float alpha = fast_exp2(run_max[nt] - safe_max);
-            run_max[nt] = next_max;
-            float tile_sum = 0.0f;
-#pragma unroll
-            for (int rt = 0; rt < RT; ++rt) {
-                float e[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    e[i] = fast_exp2(__builtin_fmaf(s[rt][nt][i], p.scale_log2e, -safe_max));
-                    tile_sum += e[i];
-                }
-                p_bits[rt][nt][0] = pack_bf16x2(e[0], e[1]);
-                p_bits[rt][nt][1] = pack_bf16x2(e[2], e[3]);
-                if (precise) {
-                    p_low[rt][nt][0] = pack_bf16x2(e[0] - bf16_bits_to_f32(p_bits[rt][nt][0] & 0xffffu), e[1] - bf16_bits_to_f32(p_bits[rt][nt][0] >> 16));
-                    p_low[rt][nt][1] = pack_bf16x2(e[2] - bf16_bits_to_f32(p_bits[rt][nt][1] & 0xffffu), e[3] - bf16_bits_to_f32(p_bits[rt][nt][1] >> 16));
-                }
-            }
-            run_sum[nt] = run_sum[nt] * alpha + tile_sum;
-            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) acc[nt][mt] *= alpha;
-            }
-        }
-        // O^T += V^T . P^T, 32 tokens per MFMA: k = 8g + j <-> token (j < 4 ? 4g + j : 16 + 4g + j - 4) of the 32-token pair.
-#pragma unroll
-        for (int pair = 0; pair < RT / 2; ++pair) {
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const unsigned char* column = v_src + (pair * 32 + g * 4 + (r16 >> 2)) * Smem::kRowBytes + (mt * 16 + (r16 & 3) * 4) * 2;
-                const s16x4v lo = lds_read_tr16(column);
-                const s16x4v hi = lds_read_tr16(column + 16 * Smem::kRowBytes);
-                const uint4 a_bits = make_uint4(__builtin_bit_cast(uint2, lo).x, __builtin_bit_cast(uint2, lo).y,
-                                                __builtin_bit_cast(uint2, hi).x, __builtin_bit_cast(uint2, hi).y);
-                const bf16x8 a = __builtin_bit_cast(bf16x8, a_bits);
-#pragma unroll
-                for (int nt = 0; nt < NTW; ++nt) {
-                    const uint4 b_bits = make_uint4(p_bits[2 * pair][nt][0], p_bits[2 * pair][nt][1], p_bits[2 * pair + 1][nt][0],
-                                                    p_bits[2 * pair + 1][nt][1]);
-                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, b_bits), acc[nt][mt], 0, 0, 0);
-                    if (precise) {
-                        const uint4 low_bits = make_uint4(p_low[2 * pair][nt][0], p_low[2 * pair][nt][1], p_low[2 * pair + 1][nt][0],
-                                                          p_low[2 * pair + 1][nt][1]);
-                        acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, low_bits), acc[nt][mt], 0, 0, 0);
-                    }
-                }
+                    out.s[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, q_frag[nt][ks]), out.s[rt][nt], 0, 0, 0);
             }
         }
     };
 
-    // ---- main loop: registers hold tile i+1 while LDS stage i%2 is consumed -------------------------------------
-    if (num_tiles > 0) {
-        load_tile(0);
-        store_tile(0, 0);
-        if (num_tiles > 1) load_tile(1);
-        for (uint32_t tile = 0; tile < num_tiles; ++tile) {
-            __syncthreads();  // stage tile%2 is complete; nobody still reads stage (tile+1)%2
-            if (tile + 1 < num_tiles) store_tile(tile + 1, (tile + 1) & 1);
-            if (tile + 2 < num_tiles) {
-                refresh_ids(tile + 2);
-                load_tile(tile + 2);
+    // One slice: S^T, softmax update, P.V.  Nothing is pipelined inside a wave; the other wave of the SIMD fills the gaps.
+    auto process_slice = [&](auto precise_tag, auto masked_tag, uint32_t slice_first, const unsigned char* k_src,
+                             const unsigned char* v_src) __attribute__((always_inline)) {
+        constexpr bool PRECISE = decltype(precise_tag)::value;
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        Scores scores;
+        scores_of(k_src, scores);
+        uint32_t p_bits[NTW][4], p_low[PRECISE ? NTW : 1][4];
+        bool rescale = false;
+        float alpha[NTW], slice_sum[NTW];
+        f32x4 (&s)[2][NTW] = scores.s;
+#pragma unroll
+        for (int nt = 0; nt < NTW; ++nt) {
+            slice_sum[nt] = 0.0f;
+            if constexpr (MASKED) {
+#pragma unroll
+                for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const uint32_t token = slice_first + rt * 16 + g * 4 + i;
+                        s[rt][nt][i] = (token >= col_lo[nt] && token < col_hi[nt]) ? s[rt][nt][i] : -INFINITY;
+                    }
             }
-            compute_tile(tile, tile & 1);
+            float tile_max = fmaxf(fmaxf(fmaxf(s[0][nt][0], s[0][nt][1]), fmaxf(s[0][nt][2], s[0][nt][3])),
+                                   fmaxf(fmaxf(s[1][nt][0], s[1][nt][1]), fmaxf(s[1][nt][2], s[1][nt][3])));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
+            tile_max *= p.scale_log2e;                                 // scale > 0: max commutes with the scaling
+            top_max[nt] = fmaxf(top_max[nt], tile_max);
+            // move the reference only when it is unset or more than the threshold below the new maximum
+            const bool move = tile_max > ref_max[nt] + kRescaleThreshold || (ref_max[nt] == -INFINITY && tile_max > -INFINITY);
+            const float next_ref = move ? tile_max : ref_max[nt];
+            alpha[nt] = move ? fast_exp2(ref_max[nt] - next_ref) : 1.0f;
+            ref_max[nt] = next_ref;
+            rescale = rescale || move;
+            const float safe_ref = next_ref == -INFINITY ? 0.0f : next_ref;
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+                float e[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) e[i] = fast_exp2(__builtin_fmaf(s[rt][nt][i], p.scale_log2e, -safe_ref));
+                slice_sum[nt] += (e[0] + e[1]) + (e[2] + e[3]);
+                p_bits[nt][2 * rt] = pack_bf16x2(e[0], e[1]);
+                p_bits[nt][2 * rt + 1] = pack_bf16x2(e[2], e[3]);
+                if constexpr (PRECISE) {
+                    p_low[nt][2 * rt] = pack_bf16x2(e[0] - bf16_bits_to_f32(p_bits[nt][2 * rt] & 0xffffu), e[1] - bf16_bits_to_f32(p_bits[nt][2 * rt] >> 16));
+                    p_low[nt][2 * rt + 1] = pack_bf16x2(e[2] - bf16_bits_to_f32(p_bits[nt][2 * rt + 1] & 0xffffu), e[3] - bf16_bits_to_f32(p_bits[nt][2 * rt + 1] >> 16));
+                }
+            }
+        }
+        if (__builtin_amdgcn_ballot_w64(rescale) != 0) {
+#pragma unroll
+            for (int nt = 0; nt < NTW; ++nt) {
+                run_sum[nt] *= alpha[nt];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[nt][mt] *= alpha[nt];
+            }
+        }
+#pragma unroll
+        for (int nt = 0; nt < NTW; ++nt) run_sum[nt] += slice_sum[nt];
+        // O^T += V^T . P^T over the 32 tokens: k = 8g + j <-> token (j < 4 ? 4g + j : 16 + 4g + j - 4) of the slice.
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const unsigned char* address = v_src + v_base + (((mt * 2) ^ v_swizzle) << 4);
+            const uint2 lo = __builtin_bit_cast(uint2, lds_read_tr16(address));
+            const uint2 hi = __builtin_bit_cast(uint2, lds_read_tr16(address + 16 * ROW));
+            const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
+#pragma unroll
+            for (int nt = 0; nt < NTW; ++nt) {
+                const uint4 b_bits = make_uint4(p_bits[nt][0], p_bits[nt][1], p_bits[nt][2], p_bits[nt][3]);
+                acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, b_bits), acc[nt][mt], 0, 0, 0);
+                if constexpr (PRECISE) {
+                    const uint4 low_bits = make_uint4(p_low[nt][0], p_low[nt][1], p_low[nt][2], p_low[nt][3]);
+                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, low_bits), acc[nt][mt], 0, 0, 0);
+                }
+            }
+        }
+    };
+    auto run_slice = [&](uint32_t slice, const unsigned char* k_src, const unsigned char* v_src) __attribute__((always_inline)) {
+        const uint32_t slice_first = first_token + slice * 32;
+        const bool interior = slice_first >= wave_all_lo && slice_first + 32 <= wave_all_hi;
+        if (precise) {
+            if (interior) process_slice(std::true_type{}, std::false_type{}, slice_first, k_src, v_src);
+            else process_slice(std::true_type{}, std::true_type{}, slice_first, k_src, v_src);
+        } else {
+            if (interior) process_slice(std::false_type{}, std::false_type{}, slice_first, k_src, v_src);
+            else process_slice(std::false_type{}, std::true_type{}, slice_first, k_src, v_src);
+        }
+    };
+
+    // ---- main loop --------------------------------------------------------------------------------------------------
+    // Tile j lives in stage j % NSTAGES.  At the top of tile j the wave waits for its own loads of tile j and the
+    // barrier publishes them; every wave has then left tile j-1, whose stage receives tile j + NSTAGES - 1.
+    if (num_tiles > 0) {
+#pragma unroll
+        for (int t = 0; t < NSTAGES - 1; ++t)
+            if ((uint32_t)t < num_tiles) issue_tile(t, fetch_ids(t));
+        TileIds upcoming = fetch_ids(NSTAGES - 1);
+        for (uint32_t tile = 0; tile < num_tiles; ++tile) {
+            // loads issued after those of this tile: tiles tile + 1 .. min(tile + NSTAGES - 2, num_tiles - 1)
+            const uint32_t last_issued = tile + NSTAGES - 2 < num_tiles - 1 ? tile + NSTAGES - 2 : num_tiles - 1;
+            const uint32_t newer = last_issued - tile;
+            if (NSTAGES >= 5 && newer >= 3) wait_vmem_outstanding<3 * LPW>();
+            else if (NSTAGES >= 4 && newer >= 2) wait_vmem_outstanding<2 * LPW>();
+            else if (newer >= 1) wait_vmem_outstanding<LPW>();
+            else wait_vmem_outstanding<0>();
+            __syncthreads();
+            if (tile + NSTAGES - 1 < num_tiles) {
+                issue_tile(tile + NSTAGES - 1, upcoming);
+                upcoming = fetch_ids(tile + NSTAGES);
+            }
+            const unsigned char* k_tile = k_lds + (tile % NSTAGES) * Smem::kTileBytes;
+            const unsigned char* v_tile = v_lds + (tile % NSTAGES) * Smem::kTileBytes;
+#pragma unroll 1
+            for (int k = 0; k < SL; ++k) {
+                const uint32_t slice = tile * SL + k;
+                if (slice < num_slices) run_slice(slice, k_tile + k * 32 * ROW, v_tile + k * 32 * ROW);
+            }
         }
     }
 
@@ -389,20 +444,21 @@ __global__ __launch_bounds__(NWAVES * 64) void tile_map_kernel(const MapParams p
     const uint32_t mode = p.output_mode;
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt) {
+        // the lanes of a column each hold the sum over their tokens, relative to ref_max
         float total = run_sum[nt];
         total += __shfl_xor(total, 16);
         total += __shfl_xor(total, 32);
         if (!col_active[nt]) continue;
         const float inverse = total > 0.0f ? 1.0f / total : 0.0f;
-        const uint32_t q_head = first_q_head + col_head[nt];
+        const uint32_t q_head = first_q_head + column_head(nt);
         uint64_t row;
         if (mode == kMapDirectBf16) {
-            row = (uint64_t)(flat_begin + col_token[nt]) * p.num_q_heads + q_head;
+            row = (uint64_t)(flat_begin + column_token(nt)) * p.num_q_heads + q_head;
         } else {
-            row = ((uint64_t)task * p.num_q_heads + q_head) * p.max_q_tokens + col_token[nt];
+            row = ((uint64_t)task * p.num_q_heads + q_head) * p.max_q_tokens + column_token(nt);
             if (g == 0) {
-                p.exp_sums[row] = total;
-                p.max_logits[row] = total > 0.0f ? run_max[nt] * 0.6931471805599453f : -INFINITY;
+                p.exp_sums[row] = total > 0.0f ? total * fast_exp2(ref_max[nt] - top_max[nt]) : 0.0f;
+                p.max_logits[row] = total > 0.0f ? top_max[nt] * 0.6931471805599453f : -INFINITY;
             }
         }
 #pragma unroll
