@@ -397,27 +397,14 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             }
         }
     };
-    auto run_slice = [&](uint32_t slice, const unsigned char* k_src, const unsigned char* v_src) __attribute__((always_inline)) {
-        const uint32_t slice_first = first_token + slice * 32;
-        const bool interior = slice_first >= wave_all_lo && slice_first + 32 <= wave_all_hi;
-        if (precise) {
-            if (interior) process_slice(std::true_type{}, std::false_type{}, slice_first, k_src, v_src);
-            else process_slice(std::true_type{}, std::true_type{}, slice_first, k_src, v_src);
-        } else {
-            if (interior) process_slice(std::false_type{}, std::false_type{}, slice_first, k_src, v_src);
-            else process_slice(std::false_type{}, std::true_type{}, slice_first, k_src, v_src);
-        }
-    };
-
     // ---- main loop --------------------------------------------------------------------------------------------------
     // Tile j lives in stage j % NSTAGES.  At the top of tile j the wave waits for its own loads of tile j and the
     // barrier publishes them; every wave has then left tile j-1, whose stage receives tile j + NSTAGES - 1.
-    if (num_tiles > 0) {
-#pragma unroll
-        for (int t = 0; t < NSTAGES - 1; ++t)
-            if ((uint32_t)t < num_tiles) issue_tile(t, fetch_ids(t));
-        TileIds upcoming = fetch_ids(NSTAGES - 1);
-        for (uint32_t tile = 0; tile < num_tiles; ++tile) {
+    // The wave walks its tiles in three runs - masked head, interior, masked tail - so that every loop holds exactly one
+    // variant of the slice code; all waves pass the same number of barriers whatever their split.
+    TileIds upcoming = fetch_ids(NSTAGES - 1);
+    auto run_tiles = [&](auto precise_tag, auto masked_tag, uint32_t tile_begin, uint32_t tile_end) __attribute__((always_inline)) {
+        for (uint32_t tile = tile_begin; tile < tile_end; ++tile) {
             // loads issued after those of this tile: tiles tile + 1 .. min(tile + NSTAGES - 2, num_tiles - 1)
             const uint32_t last_issued = tile + NSTAGES - 2 < num_tiles - 1 ? tile + NSTAGES - 2 : num_tiles - 1;
             const uint32_t newer = last_issued - tile;
@@ -432,11 +419,32 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             }
             const unsigned char* k_tile = k_lds + (tile % NSTAGES) * Smem::kTileBytes;
             const unsigned char* v_tile = v_lds + (tile % NSTAGES) * Smem::kTileBytes;
-#pragma unroll 1
+#pragma unroll
             for (int k = 0; k < SL; ++k) {
                 const uint32_t slice = tile * SL + k;
-                if (slice < num_slices) run_slice(slice, k_tile + k * 32 * ROW, v_tile + k * 32 * ROW);
+                if (k == 0 || slice < num_slices)
+                    process_slice(precise_tag, masked_tag, first_token + slice * 32, k_tile + k * 32 * ROW, v_tile + k * 32 * ROW);
             }
+        }
+    };
+    if (num_tiles > 0) {
+#pragma unroll
+        for (int t = 0; t < NSTAGES - 1; ++t)
+            if ((uint32_t)t < num_tiles) issue_tile(t, fetch_ids(t));
+        // tiles [0, head_end) and [tail_begin, num_tiles) hold tokens some active column of the wave does not see
+        uint32_t head_end = wave_all_lo > first_token ? (wave_all_lo - first_token + BK - 1) / BK : 0;
+        head_end = head_end < num_tiles ? head_end : num_tiles;
+        uint32_t tail_begin = wave_all_hi > first_token ? (wave_all_hi - first_token) / BK : 0;
+        tail_begin = tail_begin < num_tiles ? tail_begin : num_tiles;
+        tail_begin = tail_begin > head_end ? tail_begin : head_end;
+        if (precise) {
+            run_tiles(std::true_type{}, std::true_type{}, 0, head_end);
+            run_tiles(std::true_type{}, std::false_type{}, head_end, tail_begin);
+            run_tiles(std::true_type{}, std::true_type{}, tail_begin, num_tiles);
+        } else {
+            run_tiles(std::false_type{}, std::true_type{}, 0, head_end);
+            run_tiles(std::false_type{}, std::false_type{}, head_end, tail_begin);
+            run_tiles(std::false_type{}, std::true_type{}, tail_begin, num_tiles);
         }
     }
 
