@@ -234,6 +234,16 @@ class Workload:
         pairs = sum(n * h + n * (n + 1) // 2 for h, n in zip(self.histories, self.q_lens))
         return 4 * spec["hq"] * spec["d"] * pairs
 
+    def map_kernel_name(self) -> str:
+        """Name of the HIP kernel the Map launch runs: one 16-column tile (decode) uses the split-KV kernel whose waves
+        share nothing, wider Q tiles the LDS-tiled kernel."""
+        coordinates = int(self.variant.map_max_q_tokens) * int(self.variant.map_max_q_heads)
+        from khalamari_amd import sdpa
+
+        if self.variant.map_kind == sdpa.MAP_SLICED_KV or coordinates <= 16:
+            return "split_kv_map_kernel"
+        return "tile_map_kernel"
+
     def step(self, i: int) -> None:
         self.launch_map(self.kv_pools[i % len(self.kv_pools)])
         if self.launch_reduce is not None:
@@ -273,6 +283,7 @@ class Workload:
             "us_per_step": ms * 1e3,
             "map_kernel_us": map_ms * 1e3,
             "map_kernel_us_median": map_ms_median * 1e3,
+            "map_kernel": self.map_kernel_name(),
             "map_kind": int(self.variant.map_kind),
             "map_tile": [int(self.variant.map_max_q_tokens), int(self.variant.map_max_q_heads)],
             "direct_output": bool(self.direct),
@@ -417,7 +428,7 @@ def main() -> int:
             "unit": "TFLOP/s" if prefill else "GB/s",
             "frac": head["roofline_frac"],
             "traffic": None,
-            "kernel": "split_kv_map_kernel",
+            "kernel": head["map_kernel"],
             "kernel_us": head["map_kernel_us"],
             "algorithmic_bytes": head.get("algorithmic_bytes"),
             "algorithmic_flops": head.get("algorithmic_flops"),

@@ -46,9 +46,12 @@ struct TileKernelChoice {
     uint32_t smem_bytes;
 };
 
-// Tiled (LDS-shared K/V) kernel for Q tiles of 65..256 coordinates.
+// Tiled (LDS-shared K/V) kernel for Q tiles of 17..256 coordinates: speculative-verify blocks (one 16-column tile per
+// wave, bandwidth-bound) up to prefill tiles (32 columns per wave, MFMA-bound).
 static TileKernelChoice select_tile_kernel(uint32_t head_dim, uint32_t coordinates) {
     if (head_dim == 128) {
+        if (coordinates <= 64)
+            return {tile_map_kernel<128, 1, 4, 32, 4, 2>, 256, (uint32_t)TileSmem<128, 32, 4>::kBytes};  // 64 KB: two blocks per CU
         if (coordinates <= 128) return {tile_map_kernel<128, 2, 4, 64, 4, 2>, 256, (uint32_t)TileSmem<128, 64, 4>::kBytes};
 #ifdef KHM_X_TILE_B
         return {tile_map_kernel<128, 4, 4, 64, 4, 1>, 256, (uint32_t)TileSmem<128, 64, 4>::kBytes};
@@ -57,6 +60,7 @@ static TileKernelChoice select_tile_kernel(uint32_t head_dim, uint32_t coordinat
 #endif
     }
     if (head_dim == 256) {
+        if (coordinates <= 64) return {tile_map_kernel<256, 1, 4, 32, 4, 1>, 256, (uint32_t)TileSmem<256, 32, 4>::kBytes};
         if (coordinates <= 128) return {tile_map_kernel<256, 2, 4, 32, 4, 1>, 256, (uint32_t)TileSmem<256, 32, 4>::kBytes};
         return {tile_map_kernel<256, 2, 8, 32, 4, 1>, 512, (uint32_t)TileSmem<256, 32, 4>::kBytes};
     }
@@ -146,6 +150,7 @@ struct ComputeBase {
     uint32_t map_threads;
     uint32_t map_smem_bytes;
     bool direct;
+    bool map_merges_in_kernel;  // the Map kernel can merge a row's partial states itself when its last block arrives
 };
 
 static void fill_map_geometry(const ComputeBase& c, MapParams* p) {
@@ -244,6 +249,7 @@ extern "C" int khm_sliced_kv_create(const khm_gqa_sdpa_config* config, const khm
     compute->map = select_small_tile_kernel(config->head_dim, div_ceil_u32(variant->map_max_q_heads, 16));
     compute->map_threads = kMapWaves * 64;
     compute->map_smem_bytes = 0;
+    compute->map_merges_in_kernel = true;
     compute->reduce = select_reduce_kernel(config->head_dim, false);
     if (compute->map == nullptr || compute->reduce == nullptr) {
         delete compute;
@@ -433,7 +439,9 @@ extern "C" int khm_sliced_q_create(const khm_gqa_sdpa_config* config, const khm_
         compute->map = select_small_tile_kernel(config->head_dim, div_ceil_u32(coordinates, 16));
         compute->map_threads = kMapWaves * 64;
         compute->map_smem_bytes = 0;
+        compute->map_merges_in_kernel = true;
     } else {
+        compute->map_merges_in_kernel = false;
         const TileKernelChoice choice = select_tile_kernel(config->head_dim, coordinates);
         compute->map = choice.kernel;
         compute->map_threads = choice.threads;
@@ -543,6 +551,13 @@ extern "C" int khm_sliced_q_map_reduce(const khm_sliced_q* compute, const khm_sl
     KHM_BUFFER_AT_LEAST(reduce_buffers->cu_sdpa_partial_outputs, ((uint64_t)shape.num_total_q_token_tiles + 1) * 4, "cu_sdpa_partial_outputs");
     KHM_BUFFER_AT_LEAST(reduce_buffers->output, khm_gqa_sdpa_q_bytes(&config, &shape), "output");
     KHM_BUFFER_AT_LEAST(arrival_counters, khm_sliced_q_arrival_counters_bytes(&config, &compute->variant, &shape), "arrival_counters");
+    if (!compute->map_merges_in_kernel) {
+        // the LDS-tiled Map kernel has no merge epilogue: same result from the two launches, in stream order
+        if (int s = khm_sliced_q_map(compute, map_buffers, page_table_index, num_active_tokens, num_active_q_token_tiles,
+                                     num_active_kv_splits, replay_parameters, stream))
+            return s;
+        return khm_sliced_q_reduce(compute, reduce_buffers, num_active_q_token_tiles, replay_parameters, stream);
+    }
     const FusedReduceArgs fused{static_cast<const uint32_t*>(reduce_buffers->cu_sdpa_partial_outputs.ptr),
                                 static_cast<uint32_t*>(arrival_counters.ptr), static_cast<uint16_t*>(reduce_buffers->output.ptr), nullptr};
     return launch_sliced_q_map(compute, map_buffers->q, map_buffers->kv_pages, map_buffers->req_slots, map_buffers->page_ids,
@@ -609,7 +624,9 @@ extern "C" int khm_sliced_q_reduce(const khm_sliced_q* compute, const khm_sliced
     p.head_dim = config.head_dim;
     p.max_q_tokens = compute->variant.map_max_q_tokens;
     p.partial_is_f32 = config.partial_dtype == KHM_DTYPE_F32;
-    const dim3 grid(shape.num_total_q_token_tiles, config.num_q_heads, 1);
+    KHM_REQUIRE(!mul_overflows_u32(shape.num_total_q_token_tiles, compute->variant.map_max_q_tokens),
+                "GQA SplitKV SlicedQ reduce grid exceeds the u32 domain");
+    const dim3 grid(shape.num_total_q_token_tiles * compute->variant.map_max_q_tokens, config.num_q_heads, 1);
     hipLaunchKernelGGL(compute->reduce, grid, dim3(kReduceThreads), 0, static_cast<hipStream_t>(stream), p);
     return check_launch("sliced-Q reduce");
 }

@@ -26,7 +26,8 @@ namespace khm {
 constexpr int kReduceThreads = 256;
 
 // RANGED = false: sliced-KV flat reduce, grid (tokens, heads).
-// RANGED = true : sliced-Q reduce, grid (Q ranges, heads); loops the range's tokens.
+// RANGED = true : sliced-Q reduce, grid (Q ranges * max_q_tokens, heads): one block per token slot of a range, so the
+//                 tokens of a range reduce side by side rather than in a serial loop of dependent loads.
 template <int D, bool RANGED>
 __global__ __launch_bounds__(kReduceThreads) void split_kv_reduce_kernel(const ReduceParams p) {
     constexpr int CHUNKS = D / 4;                    // threads per row
@@ -34,7 +35,7 @@ __global__ __launch_bounds__(kReduceThreads) void split_kv_reduce_kernel(const R
     __shared__ float slice_stats[SLICES * 2];
     __shared__ __align__(16) float slice_acc[SLICES * D];
 
-    const uint32_t unit = blockIdx.x;
+    const uint32_t unit = RANGED ? blockIdx.x / p.max_q_tokens : blockIdx.x;
     if (unit >= resolve_u32(p.num_active, p.replay_parameters)) return;
     const uint32_t head = blockIdx.y;
     const uint32_t begin = p.cu_partial_outputs[unit];
@@ -49,7 +50,9 @@ __global__ __launch_bounds__(kReduceThreads) void split_kv_reduce_kernel(const R
     const int chunk = threadIdx.x % CHUNKS;
     const uint32_t slice = threadIdx.x / CHUNKS;
 
-    for (uint32_t local = 0; local < num_q; ++local) {
+    const uint32_t local = RANGED ? blockIdx.x - unit * p.max_q_tokens : 0u;
+    if (local >= num_q) return;
+    {
         MergeState state = merge_state_empty();
         if (end > begin) {
             merge_partial_slice<D, false>(state, p.max_logits, p.exp_sums, p.partial, p.partial_is_f32 != 0, begin + slice, end, SLICES, begin,
@@ -66,7 +69,6 @@ __global__ __launch_bounds__(kReduceThreads) void split_kv_reduce_kernel(const R
             const uint64_t out_index = ((uint64_t)(flat_begin + local) * p.num_q_heads + head) * D + chunk * 4;
             merge_store_output(total, p.output, p.gates, out_index);
         }
-        __syncthreads();
     }
 }
 

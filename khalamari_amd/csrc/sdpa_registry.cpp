@@ -92,7 +92,8 @@ int kernel_family(const khm_sdpa_config& config, const khm_sdpa_variant& variant
         return no("gfx950 kernels are built for 8, 16 or 32 tokens per page");
     if (kv_dtype != KHM_DTYPE_BF16) return no("gfx950 kernels are built for bf16 K/V pages");
     const uint64_t coordinates = (uint64_t)variant.map_max_q_tokens * variant.map_max_q_heads;
-    if (coordinates <= 64) return 1;
+    // one 16-column MFMA tile: the split-KV kernel (waves share nothing); wider tiles share K/V through LDS
+    if (coordinates <= 16 || (variant.map_kind == KHM_MAP_SLICED_KV && coordinates <= 64)) return 1;
     if (variant.map_kind == KHM_MAP_SLICED_KV) return no("sliced-KV blocks hold at most 64 Q heads");
     if (coordinates <= 256) return 2;
     return no("gfx950 kernels hold at most 256 (token, head) coordinates per block");

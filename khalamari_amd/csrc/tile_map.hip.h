@@ -47,10 +47,20 @@ __device__ __forceinline__ s16x4v lds_read_tr16(const unsigned char* address) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4v __attribute__((address_space(3)))*)(address));
 }
 
-// 16 bytes per lane from global memory to LDS: lane l of the wave lands at lds_base + 16 * l (lds_base is wave-uniform).
-__device__ __forceinline__ void load_to_lds_b128(const unsigned char* source, unsigned char* lds_base) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)source,
-                                     (__attribute__((address_space(3))) void*)lds_base, 16, 0, 0);
+// 16 bytes per lane from global memory to LDS: lane l of the wave reads uniform_base + lane_offset and lands at
+// lds_address + 16 * l (lds_address is wave-uniform and travels in M0).  Written as inline assembly on purpose: the
+// compiler makes every LDS read wait for all direct-to-LDS loads it knows of (it cannot tell which tile a read
+// touches), which would allow only one tile in flight; here the waits are explicit (wait_vmem_outstanding).
+__device__ __forceinline__ void load_to_lds_b128(const unsigned char* uniform_base, uint32_t lane_offset, uint32_t lds_address) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(lane_offset), "s"(uniform_base), "s"(lds_address)
+                 : "memory", "m0");
+}
+
+// Byte address of an LDS location as the hardware sees it.
+__device__ __forceinline__ uint32_t lds_address_of(const unsigned char* pointer) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) unsigned char*)pointer;
 }
 
 // Wait until at most COUNT of this wave's vector-memory operations are still in flight (they retire in order).
@@ -58,6 +68,21 @@ template <int COUNT>
 __device__ __forceinline__ void wait_vmem_outstanding() {
     static_assert(COUNT >= 0 && COUNT < 64, "vmcnt is a 6-bit counter");
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(COUNT) : "memory");
+}
+
+// Workgroup barrier for tiles that arrive through direct-to-LDS loads.  The caller has already waited (vmcnt) for
+// the loads it needs, so only this wave's LDS reads must have completed; __syncthreads() carries a fence that
+// would also drain every load still in flight and with it the whole multi-stage pipeline.
+__device__ __forceinline__ void barrier_keeping_loads_in_flight() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// A page-table entry read with a wave-uniform index.  The table does not change while the kernel runs, so it is
+// read through the constant address space: the compiler then issues a scalar load (its own counter) instead of a
+// vector load whose wait would also drain the K/V loads in flight.
+__device__ __forceinline__ uint32_t load_uniform_u32(const uint32_t* table, uint32_t index) {
+    typedef const uint32_t __attribute__((address_space(4))) * ConstantU32;
+    return ((ConstantU32)(uintptr_t)table)[index];
 }
 
 template <int D, int NTW, int NWAVES, int BK, int NSTAGES, int MIN_BLOCKS>
@@ -78,6 +103,8 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     extern __shared__ __align__(1024) unsigned char tile_smem[];
     unsigned char* k_lds = tile_smem;                                    // [NSTAGES][BK][ROW]
     unsigned char* v_lds = tile_smem + NSTAGES * Smem::kTileBytes;       // [NSTAGES][BK][ROW]
+    const uint32_t k_lds_address = lds_address_of(k_lds);
+    const uint32_t v_lds_address = lds_address_of(v_lds);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -214,6 +241,18 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         }
     }
 
+    // The Q loads have to be complete, in the compiler's eyes too, before the tile loop starts: a wait the compiler
+    // placed inside the loop would also drain the direct-to-LDS loads in flight, of which it knows nothing.
+#pragma unroll
+    for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
+            U32x4 bits = __builtin_bit_cast(U32x4, q_frag[nt][ks]);
+            asm volatile("" : "+v"(bits));
+            q_frag[nt][ks] = __builtin_bit_cast(uint4, bits);
+        }
+
     // ---- tile schedule -------------------------------------------------------------------------------------
     const uint32_t first_group = blk_lo >> 4;                                   // 16-token groups
     const uint32_t num_groups = blk_hi > blk_lo ? ((blk_hi - 1) >> 4) - first_group + 1 : 0;
@@ -241,7 +280,7 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             token = token < blk_lo ? blk_lo : token;
             token = token >= blk_hi ? blk_hi - 1 : token;
             const uint32_t page = token >> tpp_shift;
-            ids[i] = __builtin_amdgcn_readfirstlane(table[page < last_page ? page : last_page]);
+            ids[i] = load_uniform_u32(table, page < last_page ? page : last_page);
         }
         return ids;
     };
@@ -264,8 +303,8 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             const uint32_t in_page = (token & (tpp - 1)) * ROW;
             const uint32_t k_offset_bytes = in_page + ((load_pos ^ (row & 15)) << 4);
             const uint32_t v_offset_bytes = in_page + ((load_pos ^ ((row & 7) << 1)) << 4);
-            load_to_lds_b128(page + plane_k + k_offset_bytes, k_lds + stage * Smem::kTileBytes + unit * 1024);
-            load_to_lds_b128(page + plane_v + v_offset_bytes, v_lds + stage * Smem::kTileBytes + unit * 1024);
+            load_to_lds_b128(page + plane_k, k_offset_bytes, k_lds_address + stage * Smem::kTileBytes + unit * 1024);
+            load_to_lds_b128(page + plane_v, v_offset_bytes, v_lds_address + stage * Smem::kTileBytes + unit * 1024);
         }
     };
 
@@ -412,7 +451,7 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             else if (NSTAGES >= 4 && newer >= 2) wait_vmem_outstanding<2 * LPW>();
             else if (newer >= 1) wait_vmem_outstanding<LPW>();
             else wait_vmem_outstanding<0>();
-            __syncthreads();
+            barrier_keeping_loads_in_flight();
             if (tile + NSTAGES - 1 < num_tiles) {
                 issue_tile(tile + NSTAGES - 1, upcoming);
                 upcoming = fetch_ids(tile + NSTAGES);
