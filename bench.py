@@ -28,6 +28,10 @@ HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 TOKENS_PER_PAGE = 16
 NUM_POOLS = 3
+# HBM bytes per Map launch from the hardware counters, (FETCH_SIZE * 2.000 + WRITE_SIZE * 1.000) KiB per dispatch:
+# two `rocprofv3 --pmc` runs per config, each counter scaled by what it reads for a plain 1 GiB copy kernel
+# (`--calibration-copy`).  The summaries with their commands are the text files under profiles/.
+MEASURED_MAP_TRAFFIC_BYTES = {2: 567_707_238, 3: 2_152_189_952, 4: 1_450_992_640, 5: 1_320_510_464}
 
 CONFIGS = {
     1: dict(name="config1: B=1 q=1 Hq32/Hkv8/D128 ctx 1024, identity pages", hq=32, hkv=8, d=128, kind="decode", kv_slice=64),
@@ -369,6 +373,20 @@ def _cpu_model() -> str:
     return "unknown"
 
 
+def calibration_copy(device, gib: int = 1) -> None:
+    """A plain elementwise copy of `gib` GiB (reads and writes every byte once): what a hardware counter reads for
+    this launch, divided by its known size, is the scale factor for the same counter on the Map kernel."""
+    import torch
+
+    source = torch.full(((gib << 30) // 4,), 1.0, dtype=torch.float32, device=device)
+    target = torch.empty_like(source)
+    for _ in range(3):
+        torch.mul(source, 1.0, out=target)   # an elementwise kernel, not a DMA blit: it shows up as a dispatch
+    torch.cuda.synchronize()
+    del source, target
+    torch.cuda.empty_cache()
+
+
 def main() -> int:
     parser = argparse.ArgumentParser(description=__doc__)
     parser.add_argument("--gpus", type=int, default=1)
@@ -377,6 +395,8 @@ def main() -> int:
     parser.add_argument("--config", type=int, default=2, help="headline config (default 2)")
     parser.add_argument("--only", action="store_true", help="time only the headline config (used for profiling runs)")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    parser.add_argument("--calibration-copy", action="store_true",
+                        help="also launch a plain 1 GiB copy kernel, the known-size reference for FETCH_SIZE / WRITE_SIZE counter runs")
     args = parser.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path shards by (sequence, KV head) with no exchange, and this build runs "
@@ -388,6 +408,8 @@ def main() -> int:
         print("bench.py needs an MI355X (no GPU visible)", file=sys.stderr)
         return 2
     device = torch.device("cuda:0")
+    if args.calibration_copy:
+        calibration_copy(device)
     headline = Workload(args.config, device)
     head = headline.report(args.steps, args.warmup)
     others = {}
@@ -427,7 +449,7 @@ def main() -> int:
             "peak": MFMA_BF16_PEAK_TFLOPS if prefill else HBM_PEAK_GBPS,
             "unit": "TFLOP/s" if prefill else "GB/s",
             "frac": head["roofline_frac"],
-            "traffic": None,
+            "traffic": MEASURED_MAP_TRAFFIC_BYTES.get(args.config),
             "kernel": head["map_kernel"],
             "kernel_us": head["map_kernel_us"],
             "algorithmic_bytes": head.get("algorithmic_bytes"),
