@@ -22,6 +22,24 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // e^x through v_exp_f32; both Reduce implementations use this one so they agree bit for bit.
 __device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
 
+// Combining one value per 16-lane row over the four rows of a wave (lanes l, l^16, l^32, l^48), result in every lane.
+// gfx950 swaps lane rows inside the VALU (v_permlane16_swap / v_permlane32_swap); a generic shuffle would go through
+// the LDS crossbar, whose result also queues behind every LDS read in flight.
+__device__ __forceinline__ float max_over_rows(float x) {
+    uint32_t bits = __float_as_uint(x);
+    auto halves = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+    bits = __float_as_uint(fmaxf(__uint_as_float(halves[0]), __uint_as_float(halves[1])));
+    halves = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+    return fmaxf(__uint_as_float(halves[0]), __uint_as_float(halves[1]));
+}
+__device__ __forceinline__ float sum_over_rows(float x) {
+    uint32_t bits = __float_as_uint(x);
+    auto halves = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+    bits = __float_as_uint(__uint_as_float(halves[0]) + __uint_as_float(halves[1]));
+    halves = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+    return __uint_as_float(halves[0]) + __uint_as_float(halves[1]);
+}
+
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     f32x2 v = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));

@@ -309,8 +309,7 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
                 }
             }
             float tile_max = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16));
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
+            tile_max = max_over_rows(tile_max);
             const float next_max = fmaxf(run_max[nt], tile_max);
             const float safe_max = next_max == -INFINITY ? 0.0f : next_max;
             const float alpha = fast_exp2(run_max[nt] - safe_max);
@@ -407,8 +406,7 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
     // ---- merge the waves of the block ------------------------------------------------------
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        run_sum[nt] += __shfl_xor(run_sum[nt], 16);
-        run_sum[nt] += __shfl_xor(run_sum[nt], 32);
+        run_sum[nt] = sum_over_rows(run_sum[nt]);
         if (g == 0) {
             stats_lds[(wave * COLS + nt * 16 + r16) * 2] = run_max[nt];
             stats_lds[(wave * COLS + nt * 16 + r16) * 2 + 1] = run_sum[nt];

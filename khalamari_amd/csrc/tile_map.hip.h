@@ -358,13 +358,15 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         }
     };
 
-    // One slice: S^T, softmax update, P.V.  Nothing is pipelined inside a wave; the other wave of the SIMD fills the gaps.
-    auto process_slice = [&](auto precise_tag, auto masked_tag, uint32_t slice_first, const unsigned char* k_src,
+    // One slice: softmax update of the pending S^T, then P.V.  The S^T of the following slice is computed first: its
+    // MFMAs depend on nothing the softmax produces, so the matrix pipe works on them while the VALU does the
+    // exponentials (a software pipeline of depth one inside every wave).
+    auto process_slice = [&](auto precise_tag, auto masked_tag, uint32_t slice_first, Scores& scores, const unsigned char* k_next,
                              const unsigned char* v_src) __attribute__((always_inline)) {
         constexpr bool PRECISE = decltype(precise_tag)::value;
         constexpr bool MASKED = decltype(masked_tag)::value;
-        Scores scores;
-        scores_of(k_src, scores);
+        Scores next;
+        scores_of(k_next, next);
         uint32_t p_bits[NTW][4], p_low[PRECISE ? NTW : 1][4];
         bool rescale = false;
         float alpha[NTW], slice_sum[NTW];
@@ -383,8 +385,7 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             }
             float tile_max = fmaxf(fmaxf(fmaxf(s[0][nt][0], s[0][nt][1]), fmaxf(s[0][nt][2], s[0][nt][3])),
                                    fmaxf(fmaxf(s[1][nt][0], s[1][nt][1]), fmaxf(s[1][nt][2], s[1][nt][3])));
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16));
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
+            tile_max = max_over_rows(tile_max);
             tile_max *= p.scale_log2e;                                 // scale > 0: max commutes with the scaling
             top_max[nt] = fmaxf(top_max[nt], tile_max);
             // move the reference only when it is unset or more than the threshold below the new maximum
@@ -435,34 +436,52 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
                 }
             }
         }
+        scores = next;
     };
     // ---- main loop --------------------------------------------------------------------------------------------------
-    // Tile j lives in stage j % NSTAGES.  At the top of tile j the wave waits for its own loads of tile j and the
+    // Tile j lives in stage j % NSTAGES.  Because a slice's S^T is computed one slice ahead, tile j + 1 has to be
+    // readable while tile j is consumed: at the top of tile j the wave waits for its own loads of tile j + 1 and the
     // barrier publishes them; every wave has then left tile j-1, whose stage receives tile j + NSTAGES - 1.
     // The wave walks its tiles in three runs - masked head, interior, masked tail - so that every loop holds exactly one
     // variant of the slice code; all waves pass the same number of barriers whatever their split.
+    auto wait_for_tile = [&](uint32_t tile) __attribute__((always_inline)) {
+        // loads issued so far reach tile min(issued_until, num_tiles - 1); those after `tile` may stay in flight
+        const uint32_t newer = num_tiles - 1 - tile < (uint32_t)(NSTAGES - 2) ? num_tiles - 1 - tile : (uint32_t)(NSTAGES - 2);
+        if (NSTAGES >= 5 && newer >= 3) wait_vmem_outstanding<3 * LPW>();
+        else if (NSTAGES >= 4 && newer >= 2) wait_vmem_outstanding<2 * LPW>();
+        else if (newer >= 1) wait_vmem_outstanding<LPW>();
+        else wait_vmem_outstanding<0>();
+    };
+    auto k_slice = [&](uint32_t slice) __attribute__((always_inline)) -> const unsigned char* {
+        return k_lds + ((slice / SL) % NSTAGES) * Smem::kTileBytes + (slice % SL) * 32 * ROW;
+    };
+    auto v_slice = [&](uint32_t slice) __attribute__((always_inline)) -> const unsigned char* {
+        return v_lds + ((slice / SL) % NSTAGES) * Smem::kTileBytes + (slice % SL) * 32 * ROW;
+    };
+    Scores pending;
     TileIds upcoming = fetch_ids(NSTAGES - 1);
     auto run_tiles = [&](auto precise_tag, auto masked_tag, uint32_t tile_begin, uint32_t tile_end) __attribute__((always_inline)) {
         for (uint32_t tile = tile_begin; tile < tile_end; ++tile) {
-            // loads issued after those of this tile: tiles tile + 1 .. min(tile + NSTAGES - 2, num_tiles - 1)
-            const uint32_t last_issued = tile + NSTAGES - 2 < num_tiles - 1 ? tile + NSTAGES - 2 : num_tiles - 1;
-            const uint32_t newer = last_issued - tile;
-            if (NSTAGES >= 5 && newer >= 3) wait_vmem_outstanding<3 * LPW>();
-            else if (NSTAGES >= 4 && newer >= 2) wait_vmem_outstanding<2 * LPW>();
-            else if (newer >= 1) wait_vmem_outstanding<LPW>();
-            else wait_vmem_outstanding<0>();
+            // at this point the loads of tiles up to tile + NSTAGES - 2 have been issued
+            if (tile + 1 < num_tiles) {
+                const uint32_t last_issued = tile + NSTAGES - 2 < num_tiles - 1 ? tile + NSTAGES - 2 : num_tiles - 1;
+                const uint32_t newer = last_issued - (tile + 1);
+                if (NSTAGES >= 5 && newer >= 2) wait_vmem_outstanding<2 * LPW>();
+                else if (newer >= 1) wait_vmem_outstanding<LPW>();
+                else wait_vmem_outstanding<0>();
+            }
             barrier_keeping_loads_in_flight();
             if (tile + NSTAGES - 1 < num_tiles) {
                 issue_tile(tile + NSTAGES - 1, upcoming);
                 upcoming = fetch_ids(tile + NSTAGES);
             }
-            const unsigned char* k_tile = k_lds + (tile % NSTAGES) * Smem::kTileBytes;
-            const unsigned char* v_tile = v_lds + (tile % NSTAGES) * Smem::kTileBytes;
 #pragma unroll
             for (int k = 0; k < SL; ++k) {
                 const uint32_t slice = tile * SL + k;
-                if (k == 0 || slice < num_slices)
-                    process_slice(precise_tag, masked_tag, first_token + slice * 32, k_tile + k * 32 * ROW, v_tile + k * 32 * ROW);
+                if (k == 0 || slice < num_slices) {
+                    const uint32_t following = slice + 1 < num_slices ? slice + 1 : slice;   // the last one recomputes itself, unused
+                    process_slice(precise_tag, masked_tag, first_token + slice * 32, pending, k_slice(following), v_slice(slice));
+                }
             }
         }
     };
@@ -470,6 +489,10 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
 #pragma unroll
         for (int t = 0; t < NSTAGES - 1; ++t)
             if ((uint32_t)t < num_tiles) issue_tile(t, fetch_ids(t));
+        // publish tile 0 and start the pipeline with the scores of the first slice
+        wait_for_tile(0);
+        barrier_keeping_loads_in_flight();
+        scores_of(k_slice(0), pending);
         // tiles [0, head_end) and [tail_begin, num_tiles) hold tokens some active column of the wave does not see
         uint32_t head_end = wave_all_lo > first_token ? (wave_all_lo - first_token + BK - 1) / BK : 0;
         head_end = head_end < num_tiles ? head_end : num_tiles;
@@ -493,8 +516,7 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     for (int nt = 0; nt < NTW; ++nt) {
         // the lanes of a column each hold the sum over their tokens, relative to ref_max
         float total = run_sum[nt];
-        total += __shfl_xor(total, 16);
-        total += __shfl_xor(total, 32);
+        total = sum_over_rows(total);
         if (!col_active[nt]) continue;
         const float inverse = total > 0.0f ? 1.0f / total : 0.0f;
         const uint32_t q_head = first_q_head + column_head(nt);
