@@ -284,22 +284,44 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         }
         return ids;
     };
-    auto issue_tile = [&](uint32_t tile, const TileIds ids) __attribute__((always_inline)) {
-        const uint32_t stage = tile % NSTAGES;
-        // The lane-dependent address parts are a handful of VALU operations; the empty asm keeps the compiler from
-        // hoisting them out of the tile loop, where they would cost registers the accumulators need.
-        uint32_t lane_now = lane;
-        asm volatile("" : "+v"(lane_now));
-        const uint32_t load_row = lane_now / CPR;       // row inside a wave load
-        const uint32_t load_pos = lane_now % CPR;       // 16-byte position inside the row
+    // Lane offsets of a wave load inside its page.  A tile that lies wholly inside [blk_lo, blk_hi) needs no clamp and,
+    // BK being a multiple of the page size, its offsets do not depend on the tile: those live in registers.
+    uint32_t k_lane_offset[UPW], v_lane_offset[UPW];
+    {
+        const uint32_t load_row = lane / CPR;       // row inside a wave load
+        const uint32_t load_pos = lane % CPR;       // 16-byte position inside the row
 #pragma unroll
         for (int i = 0; i < UPW; ++i) {
-            const uint32_t unit = wave * UPW + i;                                  // wave-uniform
-            const uint32_t row = unit * RPL + load_row;                            // row inside the tile
-            uint32_t token = first_token + tile * BK + row;
+            const uint32_t row = (wave * UPW + i) * RPL + load_row;                // row inside the tile
+            const uint32_t in_page = ((first_token + row) & (tpp - 1)) * ROW;
+            k_lane_offset[i] = in_page + ((load_pos ^ (row & 15)) << 4);
+            v_lane_offset[i] = in_page + ((load_pos ^ ((row & 7) << 1)) << 4);
+        }
+    }
+    auto issue_tile = [&](uint32_t tile, const TileIds ids) __attribute__((always_inline)) {
+        const uint32_t stage = tile % NSTAGES;
+        const uint32_t tile_token = first_token + tile * BK;
+        if (tile_token >= blk_lo && tile_token + BK <= blk_hi) {
+#pragma unroll
+            for (int i = 0; i < UPW; ++i) {
+                const uint32_t unit = wave * UPW + i;                                  // wave-uniform
+                const unsigned char* page = p.kv_pages + (uint64_t)ids[i] * p.page_bytes;   // scalar
+                load_to_lds_b128(page + plane_k, k_lane_offset[i], k_lds_address + stage * Smem::kTileBytes + unit * 1024);
+                load_to_lds_b128(page + plane_v, v_lane_offset[i], v_lds_address + stage * Smem::kTileBytes + unit * 1024);
+            }
+            return;
+        }
+        // first or last tile of the range: rows outside it are redirected, which changes their offsets
+        const uint32_t load_row = lane / CPR;
+        const uint32_t load_pos = lane % CPR;
+#pragma unroll
+        for (int i = 0; i < UPW; ++i) {
+            const uint32_t unit = wave * UPW + i;
+            const uint32_t row = unit * RPL + load_row;
+            uint32_t token = tile_token + row;
             token = token < blk_lo ? blk_lo : token;
             token = token >= blk_hi ? blk_hi - 1 : token;
-            const unsigned char* page = p.kv_pages + (uint64_t)ids[i] * p.page_bytes;   // scalar
+            const unsigned char* page = p.kv_pages + (uint64_t)ids[i] * p.page_bytes;
             const uint32_t in_page = (token & (tpp - 1)) * ROW;
             const uint32_t k_offset_bytes = in_page + ((load_pos ^ (row & 15)) << 4);
             const uint32_t v_offset_bytes = in_page + ((load_pos ^ ((row & 7) << 1)) << 4);
@@ -320,17 +342,20 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     const uint32_t v_base = v_row * ROW + (r16 & 1) * 8;
 
     // ---- online-softmax state ------------------------------------------------------------------------------
-    // ref_max is the exponent reference of a column (log2 domain); it only moves when the column's maximum has
-    // grown by more than kRescaleThreshold, so the accumulators are rescaled rarely.  top_max tracks the true maximum
-    // for the partial-state ABI; the stored exp-sum is restated against it in the epilogue.
+    // Everything is kept in the log2 domain relative to ref[nt], the exponent reference of the lane's column.  The
+    // reference only moves when a score exceeds it by more than kRescaleThreshold (or when the column sees its first
+    // visible key), so the accumulators are rescaled rarely, and - what matters more - the hot path needs no
+    // cross-lane maximum at all: each lane checks its own eight scores and one ballot decides whether any column of
+    // the wave has to move.  lane_top[nt] is the largest score this lane has seen, relative to ref[nt]; the true
+    // column maximum for the partial-state ABI is reduced across lanes once, in the epilogue.
     constexpr float kRescaleThreshold = 8.0f;
     f32x4 acc[NTW][MT];
     float run_sum[NTW];
-    float ref_max[NTW], top_max[NTW];
+    float ref[NTW], lane_top[NTW];
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt) {
-        ref_max[nt] = -INFINITY;
-        top_max[nt] = -INFINITY;
+        ref[nt] = 0.0f;
+        lane_top[nt] = -INFINITY;
         run_sum[nt] = 0.0f;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -368,39 +393,60 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         Scores next;
         scores_of(k_next, next);
         uint32_t p_bits[NTW][4], p_low[PRECISE ? NTW : 1][4];
-        bool rescale = false;
-        float alpha[NTW], slice_sum[NTW];
         f32x4 (&s)[2][NTW] = scores.s;
+        // scores relative to the column reference, the lane's maximum, and whether any column must move
+        float slice_top[NTW];
+        bool lane_wants_move = false;
 #pragma unroll
         for (int nt = 0; nt < NTW; ++nt) {
-            slice_sum[nt] = 0.0f;
-            if constexpr (MASKED) {
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float value = __builtin_fmaf(s[rt][nt][i], p.scale_log2e, -ref[nt]);
+                    if constexpr (MASKED) {
+                        const uint32_t token = slice_first + rt * 16 + g * 4 + i;
+                        value = (token >= col_lo[nt] && token < col_hi[nt]) ? value : -INFINITY;
+                    }
+                    s[rt][nt][i] = value;
+                }
+            slice_top[nt] = fmaxf(fmaxf(fmaxf(s[0][nt][0], s[0][nt][1]), fmaxf(s[0][nt][2], s[0][nt][3])),
+                                  fmaxf(fmaxf(s[1][nt][0], s[1][nt][1]), fmaxf(s[1][nt][2], s[1][nt][3])));
+            // a lane that has not seen a visible key yet cannot know whether its column has a reference
+            lane_wants_move = lane_wants_move | (slice_top[nt] > kRescaleThreshold) | (lane_top[nt] == -INFINITY);
+        }
+        if (__builtin_amdgcn_ballot_w64(lane_wants_move) != 0) {
+            // rare: agree per column (its four lanes) on the maximum, move the reference and rescale what was accumulated
+#pragma unroll
+            for (int nt = 0; nt < NTW; ++nt) {
+                const float column_top = max_over_rows(slice_top[nt]);
+                const float column_seen = max_over_rows(lane_top[nt]);
+                const bool first = column_seen == -INFINITY;
+                const bool move = column_top > kRescaleThreshold || (first && column_top > -INFINITY);
+                const float shift = move ? column_top : 0.0f;
+                const float alpha = first ? 0.0f : fast_exp2(-shift);   // nothing is accumulated before the first key
+                ref[nt] += shift;
+                lane_top[nt] -= shift;
+                slice_top[nt] -= shift;
 #pragma unroll
                 for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const uint32_t token = slice_first + rt * 16 + g * 4 + i;
-                        s[rt][nt][i] = (token >= col_lo[nt] && token < col_hi[nt]) ? s[rt][nt][i] : -INFINITY;
-                    }
+                    for (int i = 0; i < 4; ++i) s[rt][nt][i] -= shift;
+                run_sum[nt] *= alpha;
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[nt][mt] *= alpha;
             }
-            float tile_max = fmaxf(fmaxf(fmaxf(s[0][nt][0], s[0][nt][1]), fmaxf(s[0][nt][2], s[0][nt][3])),
-                                   fmaxf(fmaxf(s[1][nt][0], s[1][nt][1]), fmaxf(s[1][nt][2], s[1][nt][3])));
-            tile_max = max_over_rows(tile_max);
-            tile_max *= p.scale_log2e;                                 // scale > 0: max commutes with the scaling
-            top_max[nt] = fmaxf(top_max[nt], tile_max);
-            // move the reference only when it is unset or more than the threshold below the new maximum
-            const bool move = tile_max > ref_max[nt] + kRescaleThreshold || (ref_max[nt] == -INFINITY && tile_max > -INFINITY);
-            const float next_ref = move ? tile_max : ref_max[nt];
-            alpha[nt] = move ? fast_exp2(ref_max[nt] - next_ref) : 1.0f;
-            ref_max[nt] = next_ref;
-            rescale = rescale || move;
-            const float safe_ref = next_ref == -INFINITY ? 0.0f : next_ref;
+        }
+#pragma unroll
+        for (int nt = 0; nt < NTW; ++nt) {
+            lane_top[nt] = fmaxf(lane_top[nt], slice_top[nt]);
+            float slice_sum = 0.0f;
 #pragma unroll
             for (int rt = 0; rt < 2; ++rt) {
                 float e[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) e[i] = fast_exp2(__builtin_fmaf(s[rt][nt][i], p.scale_log2e, -safe_ref));
-                slice_sum[nt] += (e[0] + e[1]) + (e[2] + e[3]);
+                for (int i = 0; i < 4; ++i) e[i] = fast_exp2(s[rt][nt][i]);
+                slice_sum += (e[0] + e[1]) + (e[2] + e[3]);
                 p_bits[nt][2 * rt] = pack_bf16x2(e[0], e[1]);
                 p_bits[nt][2 * rt + 1] = pack_bf16x2(e[2], e[3]);
                 if constexpr (PRECISE) {
@@ -408,17 +454,8 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
                     p_low[nt][2 * rt + 1] = pack_bf16x2(e[2] - bf16_bits_to_f32(p_bits[nt][2 * rt + 1] & 0xffffu), e[3] - bf16_bits_to_f32(p_bits[nt][2 * rt + 1] >> 16));
                 }
             }
+            run_sum[nt] += slice_sum;
         }
-        if (__builtin_amdgcn_ballot_w64(rescale) != 0) {
-#pragma unroll
-            for (int nt = 0; nt < NTW; ++nt) {
-                run_sum[nt] *= alpha[nt];
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) acc[nt][mt] *= alpha[nt];
-            }
-        }
-#pragma unroll
-        for (int nt = 0; nt < NTW; ++nt) run_sum[nt] += slice_sum[nt];
         // O^T += V^T . P^T over the 32 tokens: k = 8g + j <-> token (j < 4 ? 4g + j : 16 + 4g + j - 4) of the slice.
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
@@ -514,9 +551,10 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     const uint32_t mode = p.output_mode;
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt) {
-        // the lanes of a column each hold the sum over their tokens, relative to ref_max
+        // the lanes of a column each hold the sum over their tokens, relative to ref[nt]
         float total = run_sum[nt];
         total = sum_over_rows(total);
+        const float column_top = max_over_rows(lane_top[nt]);   // the column's largest score, relative to ref[nt]
         if (!col_active[nt]) continue;
         const float inverse = total > 0.0f ? 1.0f / total : 0.0f;
         const uint32_t q_head = first_q_head + column_head(nt);
@@ -526,8 +564,8 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         } else {
             row = ((uint64_t)task * p.num_q_heads + q_head) * p.max_q_tokens + column_token(nt);
             if (g == 0) {
-                p.exp_sums[row] = total > 0.0f ? total * fast_exp2(ref_max[nt] - top_max[nt]) : 0.0f;
-                p.max_logits[row] = total > 0.0f ? top_max[nt] * 0.6931471805599453f : -INFINITY;
+                p.exp_sums[row] = total > 0.0f ? total * fast_exp2(-column_top) : 0.0f;
+                p.max_logits[row] = total > 0.0f ? (ref[nt] + column_top) * 0.6931471805599453f : -INFINITY;
             }
         }
 #pragma unroll
