@@ -325,6 +325,46 @@ uint8_t khm_bf16_to_fp8_e4m3(uint16_t bf16_bits);
 uint16_t khm_fp8_e4m3_to_bf16(uint8_t fp8_bits);
 uint16_t khm_f32_to_bf16(float value);
 float khm_bf16_to_f32(uint16_t bf16_bits);
+/* The same codec on the device, element-wise over `count` values: decode is what the Map kernels apply to FP8 pages
+ * (fp8_e4m3x8_to_bf16x8, components/metal/gqa_fp8.metal:1-25), encode is what the page writer applies
+ * (bf16_to_fp8_e4m3, components/metal/gqa_kv_page_write.metal:5-31).  `codes` must be 8-byte and `bf16_out` 16-byte
+ * aligned for the decoder. */
+int khm_fp8_e4m3_to_bf16_device(khm_buffer codes, khm_buffer bf16_out, uint64_t count, void* stream);
+int khm_bf16_to_fp8_e4m3_device(khm_buffer bf16_in, khm_buffer codes, uint64_t count, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * K/V page writer: components/gqa/kv_page_write.rs:60-283, gqa_kv_page_write.metal:33-110
+ * Scatters the bf16 K and V rows [W][Hkv][D] of W token writes through the page table into pages laid out
+ * [K|V][Hkv][tokens_per_page][D].  The reference writes FP8 E4M3FN pages only; kv_dtype BF16 writes 16-bit pages.
+ * ------------------------------------------------------------------------------------------ */
+/* kv_page_write::Config (kv_page_write.rs:60-66) plus the page element type. */
+typedef struct khm_kv_page_write_config {
+    uint32_t num_kv_heads;
+    uint32_t head_dim;
+    uint32_t page_bytes;
+    uint32_t dtype;    /* source tensors: KHM_DTYPE_BF16 */
+    uint32_t kv_dtype; /* pages: KHM_DTYPE_FP8_E4M3FN (reference) or KHM_DTYPE_BF16 */
+} khm_kv_page_write_config;
+/* kv_page_write::Shape (kv_page_write.rs:115-119). */
+typedef struct khm_kv_page_write_shape {
+    uint32_t num_total_token_writes;
+    khm_page_table_layout page_table_layout;
+} khm_kv_page_write_shape;
+/* kv_page_write::Buffers (kv_page_write.rs:136-145): flat_k/flat_v bf16 [W][Hkv][D], req_slots/flat_token_indices u32 [W]. */
+typedef struct khm_kv_page_write_buffers {
+    khm_buffer pages;
+    khm_buffer flat_k;
+    khm_buffer flat_v;
+    khm_buffer req_slots;
+    khm_buffer flat_token_indices;
+    khm_buffer page_ids;
+} khm_kv_page_write_buffers;
+/* Config::num_tokens_per_page (kv_page_write.rs:76-89); 0 when page_bytes is no multiple of the K/V bytes per token. */
+uint32_t khm_kv_page_write_num_tokens_per_page(const khm_kv_page_write_config* config);
+/* Compute::invoke + Invocation::record (kv_page_write.rs:160-262): one launch, enqueued on `stream`. */
+int khm_kv_page_write(const khm_kv_page_write_config* config, const khm_kv_page_write_shape* shape,
+                      const khm_kv_page_write_buffers* buffers, khm_replay_u32 num_active_token_writes,
+                      khm_replay_u32 page_table_index, const uint32_t* replay_parameters, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Executor-side host logic that feeds the component (CPU only, no HIP calls)

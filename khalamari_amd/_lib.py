@@ -164,6 +164,25 @@ class SelectionMetrics(ctypes.Structure):
     ]
 
 
+class PageTableLayoutStruct(ctypes.Structure):
+    _fields_ = [("num_req_slots", u32), ("num_gqa_layers", u32), ("num_blocks", u32), ("num_page_ids_per_block", u32)]
+
+
+class KvPageWriteConfig(ctypes.Structure):
+    """`kv_page_write::Config` plus the page element type."""
+
+    _fields_ = [("num_kv_heads", u32), ("head_dim", u32), ("page_bytes", u32), ("dtype", u32), ("kv_dtype", u32)]
+
+
+class KvPageWriteShape(ctypes.Structure):
+    _fields_ = [("num_total_token_writes", u32), ("page_table_layout", PageTableLayoutStruct)]
+
+
+class KvPageWriteBuffers(ctypes.Structure):
+    _fields_ = [("pages", Buffer), ("flat_k", Buffer), ("flat_v", Buffer), ("req_slots", Buffer), ("flat_token_indices", Buffer),
+                ("page_ids", Buffer)]
+
+
 # Every symbol `include/khm_gqa_sdpa.h` declares; checked by tests/test_abi.py.
 EXPORTED_SYMBOLS = (
     "khm_last_error", "khm_version",
@@ -178,6 +197,8 @@ EXPORTED_SYMBOLS = (
     "khm_sliced_q_arrival_counters_bytes", "khm_sliced_q_map_reduce",
     "khm_gqa_activation_gate",
     "khm_bf16_to_fp8_e4m3", "khm_fp8_e4m3_to_bf16", "khm_f32_to_bf16", "khm_bf16_to_f32",
+    "khm_fp8_e4m3_to_bf16_device", "khm_bf16_to_fp8_e4m3_device",
+    "khm_kv_page_write_num_tokens_per_page", "khm_kv_page_write",
     "khm_replay_bucket_policy_create", "khm_replay_bucket_policy_destroy", "khm_replay_bucket_policy_max_capacity",
     "khm_replay_bucket_policy_buckets", "khm_replay_bucket_policy_capacity", "khm_replay_bucket_policy_capacity_allow_zero",
     "khm_request_shapes_from_batch",
@@ -251,6 +272,12 @@ def lib() -> ctypes.CDLL:
                                            ctypes.c_void_p]
     handle.khm_gqa_activation_gate.argtypes = [u32, u32, u32, u32, Buffer, Buffer, Buffer, ReplayU32, ctypes.c_void_p,
                                                ctypes.c_void_p]
+    handle.khm_fp8_e4m3_to_bf16_device.argtypes = [Buffer, Buffer, u64, ctypes.c_void_p]
+    handle.khm_bf16_to_fp8_e4m3_device.argtypes = [Buffer, Buffer, u64, ctypes.c_void_p]
+    handle.khm_kv_page_write_num_tokens_per_page.restype = u32
+    handle.khm_kv_page_write_num_tokens_per_page.argtypes = [ctypes.POINTER(KvPageWriteConfig)]
+    handle.khm_kv_page_write.argtypes = [ctypes.POINTER(KvPageWriteConfig), ctypes.POINTER(KvPageWriteShape),
+                                         ctypes.POINTER(KvPageWriteBuffers), ReplayU32, ReplayU32, ctypes.c_void_p, ctypes.c_void_p]
     _lib = handle
     return handle
 

@@ -22,6 +22,7 @@ SOURCES = [
     "selector.cpp",
     "batch_metadata.cpp",
     "components.hip",
+    "kv_page_write.hip",
 ]
 
 HIPCC_FLAGS = [

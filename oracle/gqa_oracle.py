@@ -335,6 +335,42 @@ def max_threads() -> int:
     return int(lib().khm_oracle_max_threads())
 
 
+# ---------------------------------------------------------------- page write
+
+
+def kv_page_write(pages, flat_k_bits, flat_v_bits, req_slots, flat_token_indices, page_ids, num_active_token_writes: int,
+                  layer: int, num_gqa_layers: int, num_blocks: int, num_page_ids_per_block: int, num_kv_heads: int,
+                  head_dim: int, tokens_per_page: int, page_bytes: int, fp8_pages: bool) -> np.ndarray:
+    """Restatement of gqa_kv_page_write_impl (components/metal/gqa_kv_page_write.metal:33-80): every active write
+    scatters its K and V rows through the page table into `[K|V][Hkv][tokens_per_page][D]` pages.
+
+    `pages` is a uint8 array [num_pages * page_bytes] and is returned modified in a copy; `flat_*_bits` are bf16 bit
+    patterns [W, Hkv, D].  FP8 pages store `bf16_bits_to_fp8` codes (the reference), bf16 pages the bits themselves.
+    """
+    out = np.array(pages, dtype=np.uint8, copy=True).reshape(-1)
+    element = 1 if fp8_pages else 2
+    k = np.asarray(flat_k_bits, dtype=np.uint16).reshape(-1, num_kv_heads, head_dim)
+    v = np.asarray(flat_v_bits, dtype=np.uint16).reshape(-1, num_kv_heads, head_dim)
+    table = np.asarray(page_ids, dtype=np.uint32).reshape(-1)
+    values_per_plane = num_kv_heads * tokens_per_page * head_dim
+    for write in range(num_active_token_writes):
+        req_slot = int(req_slots[write])
+        token = int(flat_token_indices[write])
+        block = token // (tokens_per_page * num_page_ids_per_block)
+        page_index = (token // tokens_per_page) % num_page_ids_per_block
+        page_id = int(table[((req_slot * num_gqa_layers + layer) * num_blocks + block) * num_page_ids_per_block + page_index])
+        page_token = token % tokens_per_page
+        for head in range(num_kv_heads):
+            offset = (head * tokens_per_page + page_token) * head_dim
+            for plane, row in ((0, k[write, head]), (1, v[write, head])):
+                begin = page_id * page_bytes + (plane * values_per_plane + offset) * element
+                if fp8_pages:
+                    out[begin:begin + head_dim] = bf16_bits_to_fp8(row)
+                else:
+                    out[begin:begin + 2 * head_dim] = row.view(np.uint8)
+    return out
+
+
 # ---------------------------------------------------------------- page packing (test helper)
 
 
