@@ -21,23 +21,30 @@ constexpr int kMapWaves = KHM_MAP_WAVES;
 typedef void (*MapKernel)(const MapParams);
 typedef void (*ReduceKernel)(const ReduceParams);
 
-static MapKernel select_small_tile_kernel(uint32_t head_dim, uint32_t column_tiles) {
+template <bool KV8>
+static MapKernel small_tile_kernel_of(uint32_t head_dim, uint32_t column_tiles) {
     if (head_dim == 128) {
         switch (column_tiles) {
-            case 1: return split_kv_map_kernel<128, 1, kMapWaves>;
-            case 2: return split_kv_map_kernel<128, 2, kMapWaves>;
-            case 3: return split_kv_map_kernel<128, 3, kMapWaves>;
-            case 4: return split_kv_map_kernel<128, 4, kMapWaves>;
+            case 1: return split_kv_map_kernel<128, 1, kMapWaves, KV8>;
+            case 2: return split_kv_map_kernel<128, 2, kMapWaves, KV8>;
+            case 3: return split_kv_map_kernel<128, 3, kMapWaves, KV8>;
+            case 4: return split_kv_map_kernel<128, 4, kMapWaves, KV8>;
         }
     } else if (head_dim == 256) {
         switch (column_tiles) {
-            case 1: return split_kv_map_kernel<256, 1, kMapWaves>;
-            case 2: return split_kv_map_kernel<256, 2, kMapWaves>;
-            case 3: return split_kv_map_kernel<256, 3, kMapWaves>;
-            case 4: return split_kv_map_kernel<256, 4, kMapWaves>;
+            case 1: return split_kv_map_kernel<256, 1, kMapWaves, KV8>;
+            case 2: return split_kv_map_kernel<256, 2, kMapWaves, KV8>;
+            case 3: return split_kv_map_kernel<256, 3, kMapWaves, KV8>;
+            case 4: return split_kv_map_kernel<256, 4, kMapWaves, KV8>;
         }
     }
     return nullptr;
+}
+
+// Split-KV kernel (waves share nothing) for up to 64 Q coordinates; K/V pages bf16 or FP8 E4M3FN.
+static MapKernel select_small_tile_kernel(uint32_t head_dim, uint32_t column_tiles, uint32_t kv_dtype) {
+    return kv_dtype == KHM_DTYPE_FP8_E4M3FN ? small_tile_kernel_of<true>(head_dim, column_tiles)
+                                            : small_tile_kernel_of<false>(head_dim, column_tiles);
 }
 
 struct TileKernelChoice {
@@ -246,7 +253,7 @@ extern "C" int khm_sliced_kv_create(const khm_gqa_sdpa_config* config, const khm
     compute->tokens_per_page = sdpa.tokens_per_page;
     compute->num_q_head_ranges = div_ceil_u32(sdpa.num_q_heads / sdpa.num_kv_heads, variant->map_max_q_heads);
     compute->direct = false;
-    compute->map = select_small_tile_kernel(config->head_dim, div_ceil_u32(variant->map_max_q_heads, 16));
+    compute->map = select_small_tile_kernel(config->head_dim, div_ceil_u32(variant->map_max_q_heads, 16), config->kv_dtype);
     compute->map_threads = kMapWaves * 64;
     compute->map_smem_bytes = 0;
     compute->map_merges_in_kernel = true;
@@ -436,7 +443,7 @@ extern "C" int khm_sliced_q_create(const khm_gqa_sdpa_config* config, const khm_
     compute->direct = direct_output != 0;
     const uint32_t coordinates = variant->map_max_q_tokens * variant->map_max_q_heads;
     if (family == 1) {
-        compute->map = select_small_tile_kernel(config->head_dim, div_ceil_u32(coordinates, 16));
+        compute->map = select_small_tile_kernel(config->head_dim, div_ceil_u32(coordinates, 16), config->kv_dtype);
         compute->map_threads = kMapWaves * 64;
         compute->map_smem_bytes = 0;
         compute->map_merges_in_kernel = true;

@@ -28,14 +28,22 @@
 
 #include "device_math.hip.h"
 #include "device_params.h"
+#include "fp8_device.hip.h"
 #include "lse_merge.hip.h"
 
 namespace khm {
 
-template <int D>
+// One 16-token K/V tile in registers, 16 bytes per lane and load.
+//   bf16 pages: k[ks] is the A-operand fragment of k-step ks: token row (lane & 15), dims ks*32 + (lane >> 4)*8 .. +8;
+//               v[i] is a coalesced chunk: row i*(512/D) + lane/(D/8), dims (lane % (D/8))*8 .. +8.
+//   FP8 pages:  16 bytes are 16 dims, so k[j] feeds two k-steps: token row (lane & 15), dims j*64 + (lane >> 4)*16 .. +16,
+//               the low eight for k-step 2j and the high eight for k-step 2j+1 (the Q operand uses the same dim order);
+//               v[i] is row i*(1024/D) + lane/(D/16), dims (lane % (D/16))*16 .. +16.
+template <int D, bool KV8>
 struct KvTile {
-    uint4 k[D / 32];  // A-operand fragments: token row (lane & 15), dims ks*32 + (lane >> 4)*8 .. +8
-    uint4 v[D / 32];  // coalesced chunks: row i*(512/D) + lane/(D/8), dims (lane % (D/8))*8 .. +8
+    static constexpr int kLoads = KV8 ? D / 64 : D / 32;
+    uint4 k[kLoads];
+    uint4 v[kLoads];
     uint32_t first_token;
 };
 
@@ -62,13 +70,18 @@ struct MapSmem {
 #define KHM_MAP_OCCUPANCY
 #endif
 
-template <int D, int NT, int NWAVES>
+template <int D, int NT, int NWAVES, bool KV8 = false>
 __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_kernel(const MapParams p) {
     constexpr int KS = D / 32;
     constexpr int MT = D / 16;
     constexpr int COLS = NT * 16;
-    constexpr int LANES_PER_ROW = D / 8;          // 16-byte chunks per K/V row
+    constexpr int ELEMENT_BYTES = KV8 ? 1 : 2;    // K/V page element: FP8 E4M3FN or bf16
+    constexpr int ROW_BYTES = D * ELEMENT_BYTES;
+    constexpr int LANES_PER_ROW = ROW_BYTES / 16; // 16-byte chunks per K/V row
     constexpr int ROWS_PER_LOAD = 64 / LANES_PER_ROW;
+    constexpr int LOADS = KvTile<D, KV8>::kLoads;
+    // first dim of the eight that lane group g contracts in k-step ks (the K fragments above fix the order)
+    auto q_dim = [](int ks, int g) { return KV8 ? (ks >> 1) * 64 + g * 16 + (ks & 1) * 8 : ks * 32 + g * 8; };
     using Smem = MapSmem<D, NT, NWAVES>;
     constexpr bool kQInRegs = (NT == 1);
 
@@ -175,12 +188,13 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
         if (col_active[0]) {
             const uint16_t* row = p.q + ((uint64_t)(flat_begin + token_offset) * p.num_q_heads + first_q_head + local_head) * D;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) q_frag[ks] = *reinterpret_cast<const uint4*>(row + ks * 32 + g * 8);
+            for (int ks = 0; ks < KS; ++ks) q_frag[ks] = *reinterpret_cast<const uint4*>(row + q_dim(ks, g));
         }
     } else {
-        for (int index = tid; index < COLS * LANES_PER_ROW; index += NWAVES * 64) {
-            const uint32_t c = index / LANES_PER_ROW;
-            const uint32_t chunk = index - c * LANES_PER_ROW;
+        constexpr int Q_CHUNKS = D / 8;
+        for (int index = tid; index < COLS * Q_CHUNKS; index += NWAVES * 64) {
+            const uint32_t c = index / Q_CHUNKS;
+            const uint32_t chunk = index - c * Q_CHUNKS;
             const uint32_t token_offset = c / p.max_q_heads;
             const uint32_t local_head = c - token_offset * p.max_q_heads;
             uint4 value = make_uint4(0, 0, 0, 0);
@@ -201,8 +215,8 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
     const uint32_t* table = p.page_ids + ((uint64_t)req_slot * p.num_gqa_layers + layer) * p.pages_per_request_layer;
     const uint32_t tpp = p.tokens_per_page;
     const uint32_t tpp_shift = p.tokens_per_page_shift;
-    const uint64_t kv_head_row0_k = ((uint64_t)kv_head * tpp) * (D * 2);
-    const uint64_t kv_head_row0_v = ((uint64_t)(p.num_kv_heads + kv_head) * tpp) * (D * 2);
+    const uint64_t kv_head_row0_k = ((uint64_t)kv_head * tpp) * ROW_BYTES;
+    const uint64_t kv_head_row0_v = ((uint64_t)(p.num_kv_heads + kv_head) * tpp) * ROW_BYTES;
 
     // Page ids of 64 consecutive wave tiles per register; two registers alternate.
     uint32_t ids_a[2] = {0, 0}, ids_b[2] = {0, 0};
@@ -220,7 +234,7 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
     load_ids(0, ids_a);
     if (num_wave_tiles > 64) load_ids(1, ids_b);
 
-    auto load_tile = [&](uint32_t j, KvTile<D>& tile) {
+    auto load_tile = [&](uint32_t j, KvTile<D, KV8>& tile) {
         const uint32_t chunk = j >> 6;
         if ((j & 63) == 0 && chunk >= 1 && (chunk + 1) * 64 < num_wave_tiles) {
             if ((chunk + 1) & 1) load_ids(chunk + 1, ids_b); else load_ids(chunk + 1, ids_a);
@@ -242,19 +256,19 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
             const uint32_t row = r16;
             const uint32_t in_page = (first_token + row) & (tpp - 1);
             const uint64_t page = (row >= 8 ? id1 : id0);
-            const unsigned char* base = p.kv_pages + page * p.page_bytes + kv_head_row0_k + (uint64_t)in_page * (D * 2) + g * 16;
+            const unsigned char* base = p.kv_pages + page * p.page_bytes + kv_head_row0_k + (uint64_t)in_page * ROW_BYTES + g * 16;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) tile.k[ks] = *reinterpret_cast<const uint4*>(base + ks * 64);
+            for (int i = 0; i < LOADS; ++i) tile.k[i] = *reinterpret_cast<const uint4*>(base + i * 64);
         }
         {
             const uint32_t row_in_load = lane / LANES_PER_ROW;
             const uint32_t chunk_in_row = lane % LANES_PER_ROW;
 #pragma unroll
-            for (int i = 0; i < KS; ++i) {
+            for (int i = 0; i < LOADS; ++i) {
                 const uint32_t row = i * ROWS_PER_LOAD + row_in_load;
                 const uint32_t in_page = (first_token + row) & (tpp - 1);
                 const uint64_t page = (row >= 8 ? id1 : id0);
-                const unsigned char* source = p.kv_pages + page * p.page_bytes + kv_head_row0_v + (uint64_t)in_page * (D * 2) + chunk_in_row * 16;
+                const unsigned char* source = p.kv_pages + page * p.page_bytes + kv_head_row0_v + (uint64_t)in_page * ROW_BYTES + chunk_in_row * 16;
                 tile.v[i] = *reinterpret_cast<const uint4*>(source);
             }
         }
@@ -272,7 +286,7 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
     }
     unsigned char* v_lds = v_lds_all + wave * 16 * Smem::kVRowBytes;
 
-    auto compute_tile = [&](const KvTile<D>& tile) {
+    auto compute_tile = [&](const KvTile<D, KV8>& tile) {
         const uint32_t first_token = tile.first_token;
         // S^T = K . Q^T
         f32x4 s[NT];
@@ -280,14 +294,21 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
         for (int nt = 0; nt < NT; ++nt) s[nt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            const bf16x8 a = __builtin_bit_cast(bf16x8, tile.k[ks]);
+            uint4 k_bits;
+            if constexpr (KV8) {
+                const uint4 codes = tile.k[ks >> 1];
+                k_bits = fp8x8_to_bf16x8((ks & 1) ? make_uint2(codes.z, codes.w) : make_uint2(codes.x, codes.y));
+            } else {
+                k_bits = tile.k[ks];
+            }
+            const bf16x8 a = __builtin_bit_cast(bf16x8, k_bits);
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 uint4 b_bits;
                 if constexpr (kQInRegs) {
                     b_bits = q_frag[ks];
                 } else {
-                    b_bits = *reinterpret_cast<const uint4*>(q_lds + (nt * 16 + r16) * Smem::kQRowBytes + (ks * 32 + g * 8) * 2);
+                    b_bits = *reinterpret_cast<const uint4*>(q_lds + (nt * 16 + r16) * Smem::kQRowBytes + q_dim(ks, g) * 2);
                 }
                 s[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, b_bits), s[nt], 0, 0, 0);
             }
@@ -334,16 +355,27 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
             const uint32_t chunk_in_row = lane % LANES_PER_ROW;
             const bool edge = first_token < blk_lo || first_token + 16 > blk_hi;
 #pragma unroll
-            for (int i = 0; i < KS; ++i) {
+            for (int i = 0; i < LOADS; ++i) {
                 const uint32_t row = i * ROWS_PER_LOAD + row_in_load;
                 uint4 value = tile.v[i];
                 if (edge) {
                     const uint32_t token = first_token + row;
                     if (token < blk_lo || token >= blk_hi) value = make_uint4(0, 0, 0, 0);
                 }
-                uint2* target = reinterpret_cast<uint2*>(v_lds + row * Smem::kVRowBytes + chunk_in_row * 16);
-                target[0] = make_uint2(value.x, value.y);
-                target[1] = make_uint2(value.z, value.w);
+                if constexpr (KV8) {
+                    // sixteen codes -> sixteen bf16: the staged tile is bf16 whatever the page format
+                    const uint4 low = fp8x8_to_bf16x8(make_uint2(value.x, value.y));
+                    const uint4 high = fp8x8_to_bf16x8(make_uint2(value.z, value.w));
+                    uint2* target = reinterpret_cast<uint2*>(v_lds + row * Smem::kVRowBytes + chunk_in_row * 32);
+                    target[0] = make_uint2(low.x, low.y);
+                    target[1] = make_uint2(low.z, low.w);
+                    target[2] = make_uint2(high.x, high.y);
+                    target[3] = make_uint2(high.z, high.w);
+                } else {
+                    uint2* target = reinterpret_cast<uint2*>(v_lds + row * Smem::kVRowBytes + chunk_in_row * 16);
+                    target[0] = make_uint2(value.x, value.y);
+                    target[1] = make_uint2(value.z, value.w);
+                }
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -373,7 +405,7 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
     // ---- main loop: three rotating register buffers, loads two tiles ahead -----------------
     if (num_wave_tiles > 0) {
 #if KHM_MAP_PREFETCH == 2
-        KvTile<D> t0, t1, t2;
+        KvTile<D, KV8> t0, t1, t2;
         load_tile(0, t0);
         if (num_wave_tiles > 1) load_tile(1, t1);
         uint32_t j = 0;
@@ -389,7 +421,7 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
             if (++j >= num_wave_tiles) break;
         }
 #else
-        KvTile<D> t0, t1;
+        KvTile<D, KV8> t0, t1;
         load_tile(0, t0);
         uint32_t j = 0;
         while (true) {

@@ -5,7 +5,7 @@ import numpy as np
 import torch
 
 from khalamari_amd import sdpa, sliced_kv, sliced_q
-from khalamari_amd._lib import DTYPE_BF16, DTYPE_F32, ReplayU32
+from khalamari_amd._lib import DTYPE_BF16, DTYPE_F32, DTYPE_FP8_E4M3FN, ReplayU32
 
 from oracle import gqa_oracle as oracle
 
@@ -26,7 +26,8 @@ def bf16_tensor_to_f32(t: torch.Tensor) -> np.ndarray:
 def component_config(w, cls, partial_dtype=DTYPE_BF16, num_req_slots=None):
     g = w.geom
     layout = sliced_kv.Layout(num_req_slots or w.num_req_slots, g.num_gqa_layers, g.num_blocks, g.num_page_ids_per_block)
-    return cls(g.num_q_heads, g.num_kv_heads, g.head_dim, g.scale, g.page_bytes, layout, DTYPE_BF16, DTYPE_BF16,
+    kv_dtype = DTYPE_FP8_E4M3FN if g.kv_dtype == oracle.KV_FP8_E4M3FN else DTYPE_BF16
+    return cls(g.num_q_heads, g.num_kv_heads, g.head_dim, g.scale, g.page_bytes, layout, DTYPE_BF16, kv_dtype,
                partial_dtype)
 
 

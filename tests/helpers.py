@@ -31,12 +31,14 @@ class Workload:
 
 def make_workload(*, num_q_heads, num_kv_heads, head_dim, tokens_per_page, histories, q_lens, seed, scale=None,
                   num_layers=1, layer=0, page_ids_per_block=1, permute=True, spare_pages=3, value_scale=1.0,
-                  garbage_bits=None, req_slot_order=None) -> Workload:
+                  garbage_bits=None, req_slot_order=None, fp8_pages=False) -> Workload:
     """Sequences r = 0..R-1 with `histories[r]` cached tokens and `q_lens[r]` new Q tokens (already in the cache).
 
     K/V/Q ~ N(0, value_scale) rounded to bf16.  Pages come from one shared pool, randomly permuted.
     `garbage_bits`, when given, fills every unused page slot (tokens past a sequence's end) with that bf16
-    pattern, e.g. 0x7fc0 (NaN), to prove masked slots never reach the output.
+    pattern, e.g. 0x7fc0 (NaN), to prove masked slots never reach the output (an FP8 code with `fp8_pages`).
+    `fp8_pages` stores K/V as FP8 E4M3FN codes; the values are quantised first, as the reference's tests do
+    before their oracle sees them (sliced_kv_test.rs:484-493).
     """
     rng = np.random.default_rng(seed)
     R = len(histories)
@@ -50,7 +52,7 @@ def make_workload(*, num_q_heads, num_kv_heads, head_dim, tokens_per_page, histo
     num_req_slots = max(slots) + 1
     geom = oracle.Geometry(num_q_heads, num_kv_heads, head_dim, tokens_per_page,
                            float(scale if scale is not None else head_dim ** -0.5), num_layers, num_blocks,
-                           page_ids_per_block)
+                           page_ids_per_block, oracle.KV_FP8_E4M3FN if fp8_pages else oracle.KV_BF16)
     table = np.full((num_req_slots, num_layers, num_blocks * page_ids_per_block), U32_MAX, dtype=np.uint32)
     sequences, page_lists = [], []
     cursor = 0
@@ -58,6 +60,8 @@ def make_workload(*, num_q_heads, num_kv_heads, head_dim, tokens_per_page, histo
         ctx = contexts[r]
         k = oracle.bf16_round(rng.standard_normal((ctx, num_kv_heads, head_dim), dtype=np.float32) * value_scale)
         v = oracle.bf16_round(rng.standard_normal((ctx, num_kv_heads, head_dim), dtype=np.float32) * value_scale)
+        if fp8_pages:
+            k, v = oracle.fp8_round_trip(k), oracle.fp8_round_trip(v)
         pages = order[cursor:cursor + pages_per_seq[r]]
         cursor += pages_per_seq[r]
         table[slots[r], layer, :pages_per_seq[r]] = pages
