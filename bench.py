@@ -69,11 +69,12 @@ def sample_lengths(index: int):
 class Workload:
     """One synthetic config resident in HBM plus its recorded launches."""
 
-    def __init__(self, index: int, device, num_pools: int = NUM_POOLS):
+    def __init__(self, index: int, device, num_pools: int = NUM_POOLS, fp8_pages: bool = False):
         import torch
 
         from khalamari_amd import batch_metadata, sdpa, sliced_kv, sliced_q
-        from khalamari_amd._lib import DTYPE_BF16, DTYPE_F32, ReplayU32
+        from khalamari_amd import kv_page_write
+        from khalamari_amd._lib import DTYPE_BF16, DTYPE_F32, DTYPE_FP8_E4M3FN, ReplayU32
         from khalamari_amd.selector import GQAReplayBucketPolicy, RequestShape, Selector
 
         spec = CONFIGS[index]
@@ -92,13 +93,23 @@ class Workload:
         for r, n in enumerate(pages_per_request):
             table[r, :n] = order[cursor:cursor + n]
             cursor += n
-        self.page_bytes = 2 * hkv * TOKENS_PER_PAGE * d * 2
+        # FP8 E4M3FN pages (the reference's cache format, 32 KiB at these geometries) or bf16 pages (the BASELINE configs)
+        self.fp8_pages = fp8_pages
+        self.kv_element_bytes = 1 if fp8_pages else 2
+        kv_dtype = DTYPE_FP8_E4M3FN if fp8_pages else DTYPE_BF16
+        self.page_bytes = 2 * hkv * TOKENS_PER_PAGE * d * self.kv_element_bytes
         generator = torch.Generator(device=device)
         generator.manual_seed(index)
-        self.kv_pools = [
-            torch.randn(pool_pages * self.page_bytes // 2, device=device, dtype=torch.float32, generator=generator).to(torch.bfloat16)
-            for _ in range(num_pools)
-        ]
+        self.kv_pools = []
+        for _ in range(num_pools):
+            values = torch.randn(pool_pages * self.page_bytes // self.kv_element_bytes, device=device, dtype=torch.float32,
+                                 generator=generator).to(torch.bfloat16)
+            if fp8_pages:
+                codes = torch.empty(values.numel(), dtype=torch.uint8, device=device)
+                kv_page_write.fp8_encode_device(values, codes, values.numel())
+                values = codes
+            self.kv_pools.append(values)
+        torch.cuda.synchronize()
         self.num_tokens = sum(self.q_lens)
         self.q = torch.randn((self.num_tokens, hq, d), device=device, dtype=torch.float32, generator=generator).to(torch.bfloat16)
         self.gates = None
@@ -146,7 +157,7 @@ class Workload:
         fused = fused and not self.direct
         self.fused = fused
         if self.variant.map_kind == sdpa.MAP_SLICED_KV:
-            config = sliced_kv.Config(hq, hkv, d, d ** -0.5, self.page_bytes, layout, DTYPE_BF16, DTYPE_BF16, partial_dtype)
+            config = sliced_kv.Config(hq, hkv, d, d ** -0.5, self.page_bytes, layout, DTYPE_BF16, kv_dtype, partial_dtype)
             kshape = sliced_kv.Shape(shape.num_total_tokens, shape.num_total_sdpa_map_task_templates)
             compute = sliced_kv.Compute(config, self.variant, kshape)
             scratch = sliced_kv.Scratch(device, config, kshape)
@@ -180,7 +191,7 @@ class Workload:
 
                 launch_reduce = None
         else:
-            config = sliced_q.Config(hq, hkv, d, d ** -0.5, self.page_bytes, layout, DTYPE_BF16, DTYPE_BF16, partial_dtype)
+            config = sliced_q.Config(hq, hkv, d, d ** -0.5, self.page_bytes, layout, DTYPE_BF16, kv_dtype, partial_dtype)
             qshape = sliced_q.Shape(shape.num_total_tokens, shape.num_total_q_token_tiles, shape.num_total_sdpa_map_task_templates)
             common = dict(q=self.q, req_slots=md.req_slots(), page_ids=self.page_table,
                           visible_kv_token_ranges=md.visible_kv_token_ranges(), q_token_ranges=md.q_token_ranges(),
@@ -227,7 +238,7 @@ class Workload:
     def algorithmic_bytes(self) -> int:
         """K/V bytes of every visible token once per sequence, plus Q, output and page-table reads."""
         spec = self.spec
-        kv = self.visible_tokens * spec["hkv"] * spec["d"] * 2 * 2
+        kv = self.visible_tokens * spec["hkv"] * spec["d"] * 2 * self.kv_element_bytes
         qo = 2 * self.num_tokens * spec["hq"] * spec["d"] * 2
         table = sum(-(-(h + n) // TOKENS_PER_PAGE) for h, n in zip(self.histories, self.q_lens)) * 4
         return kv + qo + table
@@ -283,7 +294,7 @@ class Workload:
         ms, map_ms, map_ms_median = self.time_steps(steps, warmup)
         spec = self.spec
         result = {
-            "workload": spec["name"],
+            "workload": spec["name"] + (" [FP8 E4M3FN pages]" if self.fp8_pages else ""),
             "us_per_step": ms * 1e3,
             "map_kernel_us": map_ms * 1e3,
             "map_kernel_us_median": map_ms_median * 1e3,
@@ -433,6 +444,15 @@ def main() -> int:
                 torch.cuda.empty_cache()
             except Exception as error:  # a config whose kernel is not built yet is reported, not hidden
                 others[f"config{index}"] = {"workload": CONFIGS[index]["name"], "error": str(error)}
+        # the reference's production cache format on the decode configs: half the bytes per KV token
+        for index in (2, 3):
+            try:
+                workload = Workload(index, device, fp8_pages=True)
+                others[f"config{index}_fp8_pages"] = workload.report(max(args.steps // 4, 10), max(args.warmup // 2, 3))
+                del workload
+                torch.cuda.empty_cache()
+            except Exception as error:
+                others[f"config{index}_fp8_pages"] = {"workload": CONFIGS[index]["name"] + " [FP8 E4M3FN pages]", "error": str(error)}
     prefill = head["bound"] == "mfma"
     line = {
         "metric": "paged GQA prefill bf16 MFMA TFLOP/s" if prefill else "paged GQA decode achieved HBM GB/s (split-KV Map + LSE Reduce per step)",
