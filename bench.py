@@ -444,8 +444,8 @@ def main() -> int:
                 torch.cuda.empty_cache()
             except Exception as error:  # a config whose kernel is not built yet is reported, not hidden
                 others[f"config{index}"] = {"workload": CONFIGS[index]["name"], "error": str(error)}
-        # the reference's production cache format on the decode configs: half the bytes per KV token
-        for index in (2, 3):
+        # the reference's production cache format: half the bytes per KV token
+        for index in (2, 3, 4, 5):
             try:
                 workload = Workload(index, device, fp8_pages=True)
                 others[f"config{index}_fp8_pages"] = workload.report(max(args.steps // 4, 10), max(args.warmup // 2, 3))

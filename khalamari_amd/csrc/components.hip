@@ -55,16 +55,25 @@ struct TileKernelChoice {
 
 // Tiled (LDS-shared K/V) kernel for Q tiles of 17..256 coordinates: speculative-verify blocks (one 16-column tile per
 // wave, bandwidth-bound) up to prefill tiles (32 columns per wave, MFMA-bound).
-static TileKernelChoice select_tile_kernel(uint32_t head_dim, uint32_t coordinates) {
+static TileKernelChoice select_tile_kernel(uint32_t head_dim, uint32_t coordinates, uint32_t kv_dtype) {
+    if (kv_dtype == KHM_DTYPE_FP8_E4M3FN) {
+        if (head_dim == 128) {
+            if (coordinates <= 64) return {tile_map_kernel<128, 1, 4, 32, 4, 2, true>, 256, (uint32_t)TileSmem<128, 32, 4>::kBytes};
+            if (coordinates <= 128) return {tile_map_kernel<128, 2, 4, 64, 4, 2, true>, 256, (uint32_t)TileSmem<128, 64, 4>::kBytes};
+            return {tile_map_kernel<128, 2, 8, 64, 4, 1, true>, 512, (uint32_t)TileSmem<128, 64, 4>::kBytes};
+        }
+        if (head_dim == 256) {
+            if (coordinates <= 64) return {tile_map_kernel<256, 1, 4, 32, 4, 1, true>, 256, (uint32_t)TileSmem<256, 32, 4>::kBytes};
+            if (coordinates <= 128) return {tile_map_kernel<256, 2, 4, 32, 4, 1, true>, 256, (uint32_t)TileSmem<256, 32, 4>::kBytes};
+            return {tile_map_kernel<256, 2, 8, 32, 4, 1, true>, 512, (uint32_t)TileSmem<256, 32, 4>::kBytes};
+        }
+        return {nullptr, 0, 0};
+    }
     if (head_dim == 128) {
         if (coordinates <= 64)
             return {tile_map_kernel<128, 1, 4, 32, 4, 2>, 256, (uint32_t)TileSmem<128, 32, 4>::kBytes};  // 64 KB: two blocks per CU
         if (coordinates <= 128) return {tile_map_kernel<128, 2, 4, 64, 4, 2>, 256, (uint32_t)TileSmem<128, 64, 4>::kBytes};
-#ifdef KHM_X_TILE_B
-        return {tile_map_kernel<128, 4, 4, 64, 4, 1>, 256, (uint32_t)TileSmem<128, 64, 4>::kBytes};
-#else
         return {tile_map_kernel<128, 2, 8, 64, 4, 1>, 512, (uint32_t)TileSmem<128, 64, 4>::kBytes};
-#endif
     }
     if (head_dim == 256) {
         if (coordinates <= 64) return {tile_map_kernel<256, 1, 4, 32, 4, 1>, 256, (uint32_t)TileSmem<256, 32, 4>::kBytes};
@@ -449,7 +458,7 @@ extern "C" int khm_sliced_q_create(const khm_gqa_sdpa_config* config, const khm_
         compute->map_merges_in_kernel = true;
     } else {
         compute->map_merges_in_kernel = false;
-        const TileKernelChoice choice = select_tile_kernel(config->head_dim, coordinates);
+        const TileKernelChoice choice = select_tile_kernel(config->head_dim, coordinates, config->kv_dtype);
         compute->map = choice.kernel;
         compute->map_threads = choice.threads;
         compute->map_smem_bytes = choice.smem_bytes;

@@ -92,12 +92,8 @@ int kernel_family(const khm_sdpa_config& config, const khm_sdpa_variant& variant
         return no("gfx950 kernels are built for 8, 16 or 32 tokens per page");
     if (kv_dtype != KHM_DTYPE_BF16 && kv_dtype != KHM_DTYPE_FP8_E4M3FN) return no("gfx950 kernels read bf16 or FP8 E4M3FN K/V pages");
     const uint64_t coordinates = (uint64_t)variant.map_max_q_tokens * variant.map_max_q_heads;
-    if (kv_dtype == KHM_DTYPE_FP8_E4M3FN) {
-        // FP8 pages are decoded in registers by the split-KV kernel; the LDS-tiled kernel reads bf16 pages only
-        if (coordinates <= 64) return 1;
-        return no("gfx950 kernels for FP8 E4M3FN K/V pages hold at most 64 (token, head) coordinates per block");
-    }
-    // one 16-column MFMA tile: the split-KV kernel (waves share nothing); wider tiles share K/V through LDS
+    // one 16-column MFMA tile: the split-KV kernel (waves share nothing); wider tiles share K/V through LDS.  Both
+    // kernel families read bf16 and FP8 E4M3FN pages.
     if (coordinates <= 16 || (variant.map_kind == KHM_MAP_SLICED_KV && coordinates <= 64)) return 1;
     if (variant.map_kind == KHM_MAP_SLICED_KV) return no("sliced-KV blocks hold at most 64 Q heads");
     if (coordinates <= 256) return 2;

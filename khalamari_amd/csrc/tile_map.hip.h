@@ -26,6 +26,7 @@
 
 #include "device_math.hip.h"
 #include "device_params.h"
+#include "fp8_device.hip.h"
 
 #ifndef KHM_X_PRECISE
 #define KHM_X_PRECISE true
@@ -85,18 +86,24 @@ __device__ __forceinline__ uint32_t load_uniform_u32(const uint32_t* table, uint
     return ((ConstantU32)(uintptr_t)table)[index];
 }
 
-template <int D, int NTW, int NWAVES, int BK, int NSTAGES, int MIN_BLOCKS>
+// KV8: the pages hold FP8 E4M3FN codes.  The LDS tiles stay bf16 in the same swizzled layout, so everything after the
+// load is unchanged; the tile itself travels through registers (16 bytes = 16 codes per lane and load), is decoded
+// there and written to LDS one barrier before it is first read.  One tile is in flight in registers while two are
+// consumed: enough for the MFMA-bound prefill tiles this mode is built for.
+template <int D, int NTW, int NWAVES, int BK, int NSTAGES, int MIN_BLOCKS, bool KV8 = false>
 __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const MapParams p) {
     constexpr int KS = D / 32;                      // QK k-steps
     constexpr int MT = D / 16;                      // PV dim tiles
     constexpr int SL = BK / 32;                     // slices per tile
-    constexpr int CPR = D / 8;                      // 16-byte chunks per K/V row
+    constexpr int PAGE_ROW = D * (KV8 ? 1 : 2);     // bytes of one K/V row in a page
+    constexpr int CPR = PAGE_ROW / 16;              // 16-byte chunks per K/V row in a page
     constexpr int RPL = 64 / CPR;                   // rows per wave load
     constexpr int UNITS = BK / RPL;                 // wave loads per plane and tile
     constexpr int UPW = UNITS / NWAVES;             // ... per wave
     constexpr int LPW = 2 * UPW;                    // K + V loads per wave and tile
     static_assert(UNITS % NWAVES == 0 && UPW >= 1, "tile loads must divide evenly over the waves");
     static_assert((SL == 1 || SL == 2) && NSTAGES >= 3 && NSTAGES <= 5, "unsupported tiling");
+    static_assert(!KV8 || NSTAGES == 4, "the register-staged FP8 path is written for a ring of four tiles");
     using Smem = TileSmem<D, BK, NSTAGES>;
     constexpr int ROW = Smem::kRowBytes;
 
@@ -262,8 +269,8 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     const uint32_t* table = p.page_ids + ((uint64_t)req_slot * p.num_gqa_layers + layer) * p.pages_per_request_layer;
     const uint32_t tpp = p.tokens_per_page;
     const uint32_t tpp_shift = p.tokens_per_page_shift;
-    const uint64_t plane_k = ((uint64_t)kv_head * tpp) * ROW;
-    const uint64_t plane_v = ((uint64_t)(p.num_kv_heads + kv_head) * tpp) * ROW;
+    const uint64_t plane_k = ((uint64_t)kv_head * tpp) * PAGE_ROW;
+    const uint64_t plane_v = ((uint64_t)(p.num_kv_heads + kv_head) * tpp) * PAGE_ROW;
 
     // A wave load covers RPL rows that lie inside one 8-token half of a 16-token group, before and after the clamp
     // below, so its page is wave-uniform: the page id travels through a scalar load, fetched one iteration before the
@@ -327,6 +334,42 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             const uint32_t v_offset_bytes = in_page + ((load_pos ^ ((row & 7) << 1)) << 4);
             load_to_lds_b128(page + plane_k, k_offset_bytes, k_lds_address + stage * Smem::kTileBytes + unit * 1024);
             load_to_lds_b128(page + plane_v, v_offset_bytes, v_lds_address + stage * Smem::kTileBytes + unit * 1024);
+        }
+    };
+
+    // FP8 pages: one tile in registers, decoded into the bf16 LDS layout the direct loads would have produced
+    // (source chunk c of a K row lands at position c ^ (row & 15), of a V row at c ^ 2 (row & 7)).
+    uint4 raw_k[KV8 ? UPW : 1], raw_v[KV8 ? UPW : 1];
+    auto load_raw_tile = [&](uint32_t tile, const TileIds ids) __attribute__((always_inline)) {
+        const uint32_t load_row = lane / CPR;
+        const uint32_t load_pos = lane % CPR;
+        const uint32_t tile_token = first_token + tile * BK;
+#pragma unroll
+        for (int i = 0; i < UPW; ++i) {
+            uint32_t token = tile_token + (wave * UPW + i) * RPL + load_row;
+            token = token < blk_lo ? blk_lo : token;
+            token = token >= blk_hi ? blk_hi - 1 : token;
+            const unsigned char* page = p.kv_pages + (uint64_t)ids[i] * p.page_bytes;
+            const uint32_t offset = (token & (tpp - 1)) * PAGE_ROW + load_pos * 16;
+            raw_k[i] = *reinterpret_cast<const uint4*>(page + plane_k + offset);
+            raw_v[i] = *reinterpret_cast<const uint4*>(page + plane_v + offset);
+        }
+    };
+    auto write_raw_tile = [&](uint32_t tile) __attribute__((always_inline)) {
+        const uint32_t load_row = lane / CPR;
+        const uint32_t load_pos = lane % CPR;
+        unsigned char* k_stage = k_lds + (tile % NSTAGES) * Smem::kTileBytes;
+        unsigned char* v_stage = v_lds + (tile % NSTAGES) * Smem::kTileBytes;
+#pragma unroll
+        for (int i = 0; i < UPW; ++i) {
+            const uint32_t row = (wave * UPW + i) * RPL + load_row;
+            const uint32_t k_swizzle = row & 15, v_swizzle_row = (row & 7) << 1;
+            const uint4 k_low = fp8x8_to_bf16x8(make_uint2(raw_k[i].x, raw_k[i].y)), k_high = fp8x8_to_bf16x8(make_uint2(raw_k[i].z, raw_k[i].w));
+            const uint4 v_low = fp8x8_to_bf16x8(make_uint2(raw_v[i].x, raw_v[i].y)), v_high = fp8x8_to_bf16x8(make_uint2(raw_v[i].z, raw_v[i].w));
+            *reinterpret_cast<uint4*>(k_stage + row * ROW + (((2 * load_pos) ^ k_swizzle) << 4)) = k_low;
+            *reinterpret_cast<uint4*>(k_stage + row * ROW + (((2 * load_pos + 1) ^ k_swizzle) << 4)) = k_high;
+            *reinterpret_cast<uint4*>(v_stage + row * ROW + (((2 * load_pos) ^ v_swizzle_row) << 4)) = v_low;
+            *reinterpret_cast<uint4*>(v_stage + row * ROW + (((2 * load_pos + 1) ^ v_swizzle_row) << 4)) = v_high;
         }
     };
 
@@ -499,18 +542,28 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     TileIds upcoming = fetch_ids(NSTAGES - 1);
     auto run_tiles = [&](auto precise_tag, auto masked_tag, uint32_t tile_begin, uint32_t tile_end) __attribute__((always_inline)) {
         for (uint32_t tile = tile_begin; tile < tile_end; ++tile) {
-            // at this point the loads of tiles up to tile + NSTAGES - 2 have been issued
-            if (tile + 1 < num_tiles) {
-                const uint32_t last_issued = tile + NSTAGES - 2 < num_tiles - 1 ? tile + NSTAGES - 2 : num_tiles - 1;
-                const uint32_t newer = last_issued - (tile + 1);
-                if (NSTAGES >= 5 && newer >= 2) wait_vmem_outstanding<2 * LPW>();
-                else if (newer >= 1) wait_vmem_outstanding<LPW>();
-                else wait_vmem_outstanding<0>();
-            }
-            barrier_keeping_loads_in_flight();
-            if (tile + NSTAGES - 1 < num_tiles) {
-                issue_tile(tile + NSTAGES - 1, upcoming);
-                upcoming = fetch_ids(tile + NSTAGES);
+            if constexpr (KV8) {
+                // tile + 1 was written to LDS during the previous tile; tile + 2 sits in registers, tile + 3 is requested
+                barrier_keeping_loads_in_flight();
+                if (tile + 2 < num_tiles) write_raw_tile(tile + 2);
+                if (tile + 3 < num_tiles) {
+                    load_raw_tile(tile + 3, upcoming);
+                    upcoming = fetch_ids(tile + 4);
+                }
+            } else {
+                // at this point the loads of tiles up to tile + NSTAGES - 2 have been issued
+                if (tile + 1 < num_tiles) {
+                    const uint32_t last_issued = tile + NSTAGES - 2 < num_tiles - 1 ? tile + NSTAGES - 2 : num_tiles - 1;
+                    const uint32_t newer = last_issued - (tile + 1);
+                    if (NSTAGES >= 5 && newer >= 2) wait_vmem_outstanding<2 * LPW>();
+                    else if (newer >= 1) wait_vmem_outstanding<LPW>();
+                    else wait_vmem_outstanding<0>();
+                }
+                barrier_keeping_loads_in_flight();
+                if (tile + NSTAGES - 1 < num_tiles) {
+                    issue_tile(tile + NSTAGES - 1, upcoming);
+                    upcoming = fetch_ids(tile + NSTAGES);
+                }
             }
 #pragma unroll
             for (int k = 0; k < SL; ++k) {
@@ -523,11 +576,22 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         }
     };
     if (num_tiles > 0) {
+        if constexpr (KV8) {
+            // tiles 0 and 1 into LDS, tile 2 into registers
+            load_raw_tile(0, fetch_ids(0));
+            write_raw_tile(0);
+            if (num_tiles > 1) {
+                load_raw_tile(1, fetch_ids(1));
+                write_raw_tile(1);
+            }
+            if (num_tiles > 2) load_raw_tile(2, fetch_ids(2));
+        } else {
 #pragma unroll
-        for (int t = 0; t < NSTAGES - 1; ++t)
-            if ((uint32_t)t < num_tiles) issue_tile(t, fetch_ids(t));
-        // publish tile 0 and start the pipeline with the scores of the first slice
-        wait_for_tile(0);
+            for (int t = 0; t < NSTAGES - 1; ++t)
+                if ((uint32_t)t < num_tiles) issue_tile(t, fetch_ids(t));
+            // publish tile 0 and start the pipeline with the scores of the first slice
+            wait_for_tile(0);
+        }
         barrier_keeping_loads_in_flight();
         scores_of(k_slice(0), pending);
         // tiles [0, head_end) and [tail_begin, num_tiles) hold tokens some active column of the wave does not see

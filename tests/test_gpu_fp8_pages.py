@@ -59,13 +59,29 @@ def test_fp8_spec_verify_blocks(device):
         helpers.assert_parity(actual, expected, "fp8 verify")
 
 
-def test_fp8_wide_tiles_are_reported_unsupported(device):
-    """Tiles above 64 coordinates on FP8 pages have no gfx950 kernel yet: creation fails loudly, nothing falls back."""
-    histories, q_lens = [64], [32]
-    w = helpers.make_workload(num_q_heads=16, num_kv_heads=2, head_dim=128, tokens_per_page=16, histories=histories, q_lens=q_lens,
-                              seed=35, fp8_pages=True)
-    config = gpu_runner.component_config(w, sliced_q.Config)
-    assert config.kv_dtype == DTYPE_FP8_E4M3FN
-    variant = sdpa.ExecutionVariant.sliced_q(config.sdpa_config(), sdpa.MAP_Q_TOKENS_AND_HEADS, 32, 16, 8)
-    with pytest.raises(_lib.KhmError, match="FP8 E4M3FN"):
-        sliced_q.Compute(config, variant, sliced_q.Shape(32, 1, 1))
+@pytest.mark.parametrize("hq,hkv,d,tile", [(64, 8, 128, 32), (32, 4, 128, 16), (24, 4, 256, 16), (16, 2, 256, 32)])
+def test_fp8_chunked_prefill_onto_a_paged_prefix(device, hq, hkv, d, tile):
+    """Causal chunks appended to paged prefixes on FP8 pages: wide Q tiles on the LDS-tiled kernel, whose tiles are
+    decoded on their way into LDS; direct output and split-KV + Reduce; the FP8 NaN code in every unused page slot."""
+    histories = [0, 333, 1000]
+    q_lens = [150, 64, 37]
+    w = helpers.make_workload(num_q_heads=hq, num_kv_heads=hkv, head_dim=d, tokens_per_page=16, histories=histories, q_lens=q_lens,
+                              seed=190 + tile, garbage_bits=0x7F, fp8_pages=True)
+    expected = helpers.expected_output(w)
+    for kv_slice, direct in [(1 << 20, True), (256, False), (100, False)]:
+        ranges, templates, cu = helpers.fixed_slice_plan(histories, q_lens, tile, kv_slice)
+        print(f"fp8 prefill hq={hq} hkv={hkv} d={d} tile={tile} kv_slice={kv_slice} direct={direct}", flush=True)
+        actual = gpu_runner.run_sliced_q(w, ranges, templates, cu, device, kind=sdpa.MAP_Q_TOKENS_AND_HEADS, max_q_tokens=tile,
+                                         max_q_heads=hq // hkv, stage=64, direct=direct)
+        helpers.assert_parity(actual, expected, f"fp8 prefill tile={tile} slice={kv_slice} direct={direct}")
+
+
+@pytest.mark.parametrize("tpp", [8, 32])
+def test_fp8_prefill_other_page_sizes(device, tpp):
+    histories, q_lens = [77, 0], [70, 33]
+    w = helpers.make_workload(num_q_heads=16, num_kv_heads=2, head_dim=256, tokens_per_page=tpp, histories=histories, q_lens=q_lens,
+                              seed=195 + tpp, fp8_pages=True)
+    ranges, templates, cu = helpers.fixed_slice_plan(histories, q_lens, 32, 1 << 20)
+    actual = gpu_runner.run_sliced_q(w, ranges, templates, cu, device, kind=sdpa.MAP_Q_TOKENS_AND_HEADS, max_q_tokens=32, max_q_heads=8,
+                                     stage=64, direct=True)
+    helpers.assert_parity(actual, helpers.expected_output(w), f"fp8 prefill tpp={tpp}")
