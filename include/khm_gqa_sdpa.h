@@ -367,6 +367,45 @@ int khm_kv_page_write(const khm_kv_page_write_config* config, const khm_kv_page_
                       khm_replay_u32 page_table_index, const uint32_t* replay_parameters, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Dense bidirectional block SDPA: components/gqa/bidi_block_sdpa.rs:44-340, gqa_bidi_block_sdpa.metal:10-126
+ * Every Q token attends, unmasked, to the block_size local K/V tokens of its own request block; the result is written
+ * as the LAST partial state of the token's Q range (slot cu_sdpa_partial_outputs[range + 1] - 1) in the sliced-Q
+ * partial layout, so that khm_sliced_q_reduce merges it with the history partials of khm_sliced_q_map.
+ * ------------------------------------------------------------------------------------------ */
+/* bidi_block_sdpa::Config (bidi_block_sdpa.rs:55-63). */
+typedef struct khm_bidi_block_sdpa_config {
+    uint32_t block_size;
+    uint32_t max_q_tokens;
+    uint32_t num_q_heads;
+    uint32_t num_kv_heads;
+    uint32_t head_dim;
+    float scale;
+    uint32_t dtype; /* KHM_DTYPE_F32 or KHM_DTYPE_BF16: q, local_k, local_v and partial_output */
+} khm_bidi_block_sdpa_config;
+/* bidi_block_sdpa::Shape (bidi_block_sdpa.rs:140-145). */
+typedef struct khm_bidi_block_sdpa_shape {
+    uint32_t num_total_tokens;
+    uint32_t num_total_q_token_ranges;
+    uint32_t num_total_partial_output_slots;
+} khm_bidi_block_sdpa_shape;
+/* bidi_block_sdpa::Buffers (bidi_block_sdpa.rs:175-185): q [T][Hq][D], local_k/local_v [T][Hkv][D]. */
+typedef struct khm_bidi_block_sdpa_buffers {
+    khm_buffer q;
+    khm_buffer local_k;
+    khm_buffer local_v;
+    khm_buffer q_token_ranges;
+    khm_buffer cu_sdpa_partial_outputs;
+    khm_buffer partial_exp_sums;
+    khm_buffer partial_max_logits;
+    khm_buffer partial_output;
+} khm_bidi_block_sdpa_buffers;
+/* Compute::invoke + Invocation::record (bidi_block_sdpa.rs:227-287): one launch, enqueued on `stream`.  A Fixed
+ * num_active_q_token_ranges must equal num_total_q_token_ranges, as in the reference (bidi_block_sdpa.rs:292-294). */
+int khm_bidi_block_sdpa(const khm_bidi_block_sdpa_config* config, const khm_bidi_block_sdpa_shape* shape,
+                        const khm_bidi_block_sdpa_buffers* buffers, khm_replay_u32 num_active_q_token_ranges,
+                        const uint32_t* replay_parameters, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Executor-side host logic that feeds the component (CPU only, no HIP calls)
  * ------------------------------------------------------------------------------------------ */
 

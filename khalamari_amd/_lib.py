@@ -183,6 +183,22 @@ class KvPageWriteBuffers(ctypes.Structure):
                 ("page_ids", Buffer)]
 
 
+class BidiBlockSdpaConfig(ctypes.Structure):
+    """`bidi_block_sdpa::Config`."""
+
+    _fields_ = [("block_size", u32), ("max_q_tokens", u32), ("num_q_heads", u32), ("num_kv_heads", u32), ("head_dim", u32),
+                ("scale", ctypes.c_float), ("dtype", u32)]
+
+
+class BidiBlockSdpaShape(ctypes.Structure):
+    _fields_ = [("num_total_tokens", u32), ("num_total_q_token_ranges", u32), ("num_total_partial_output_slots", u32)]
+
+
+class BidiBlockSdpaBuffers(ctypes.Structure):
+    _fields_ = [("q", Buffer), ("local_k", Buffer), ("local_v", Buffer), ("q_token_ranges", Buffer), ("cu_sdpa_partial_outputs", Buffer),
+                ("partial_exp_sums", Buffer), ("partial_max_logits", Buffer), ("partial_output", Buffer)]
+
+
 # Every symbol `include/khm_gqa_sdpa.h` declares; checked by tests/test_abi.py.
 EXPORTED_SYMBOLS = (
     "khm_last_error", "khm_version",
@@ -199,6 +215,7 @@ EXPORTED_SYMBOLS = (
     "khm_bf16_to_fp8_e4m3", "khm_fp8_e4m3_to_bf16", "khm_f32_to_bf16", "khm_bf16_to_f32",
     "khm_fp8_e4m3_to_bf16_device", "khm_bf16_to_fp8_e4m3_device",
     "khm_kv_page_write_num_tokens_per_page", "khm_kv_page_write",
+    "khm_bidi_block_sdpa",
     "khm_replay_bucket_policy_create", "khm_replay_bucket_policy_destroy", "khm_replay_bucket_policy_max_capacity",
     "khm_replay_bucket_policy_buckets", "khm_replay_bucket_policy_capacity", "khm_replay_bucket_policy_capacity_allow_zero",
     "khm_request_shapes_from_batch",
@@ -278,6 +295,8 @@ def lib() -> ctypes.CDLL:
     handle.khm_kv_page_write_num_tokens_per_page.argtypes = [ctypes.POINTER(KvPageWriteConfig)]
     handle.khm_kv_page_write.argtypes = [ctypes.POINTER(KvPageWriteConfig), ctypes.POINTER(KvPageWriteShape),
                                          ctypes.POINTER(KvPageWriteBuffers), ReplayU32, ReplayU32, ctypes.c_void_p, ctypes.c_void_p]
+    handle.khm_bidi_block_sdpa.argtypes = [ctypes.POINTER(BidiBlockSdpaConfig), ctypes.POINTER(BidiBlockSdpaShape),
+                                           ctypes.POINTER(BidiBlockSdpaBuffers), ReplayU32, ctypes.c_void_p, ctypes.c_void_p]
     _lib = handle
     return handle
 

@@ -23,6 +23,7 @@ SOURCES = [
     "batch_metadata.cpp",
     "components.hip",
     "kv_page_write.hip",
+    "bidi_block_sdpa.hip",
 ]
 
 HIPCC_FLAGS = [

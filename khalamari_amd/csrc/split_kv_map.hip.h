@@ -402,37 +402,29 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
         __builtin_amdgcn_wave_barrier();
     };
 
-    // ---- main loop: three rotating register buffers, loads two tiles ahead -----------------
+    // ---- main loop: a ring of register buffers, loads DEPTH tiles ahead ----------------------
+    // Two tiles in flight per wave (8 KB each at D 128 on bf16 pages, half that on FP8 pages, where four in flight were
+    // measured slower than two).  The ring is indexed with compile-time constants after unrolling.
+    constexpr int DEPTH = KHM_MAP_PREFETCH;
     if (num_wave_tiles > 0) {
-#if KHM_MAP_PREFETCH == 2
-        KvTile<D, KV8> t0, t1, t2;
-        load_tile(0, t0);
-        if (num_wave_tiles > 1) load_tile(1, t1);
+        KvTile<D, KV8> ring[DEPTH + 1];
+#pragma unroll
+        for (int i = 0; i < DEPTH; ++i)
+            if ((uint32_t)i < num_wave_tiles) load_tile(i, ring[i]);
         uint32_t j = 0;
-        while (true) {
-            if (j + 2 < num_wave_tiles) load_tile(j + 2, t2);
-            compute_tile(t0);
-            if (++j >= num_wave_tiles) break;
-            if (j + 2 < num_wave_tiles) load_tile(j + 2, t0);
-            compute_tile(t1);
-            if (++j >= num_wave_tiles) break;
-            if (j + 2 < num_wave_tiles) load_tile(j + 2, t1);
-            compute_tile(t2);
-            if (++j >= num_wave_tiles) break;
+        for (;;) {
+            bool finished = false;
+#pragma unroll
+            for (int slot = 0; slot <= DEPTH; ++slot) {
+                if (j + DEPTH < num_wave_tiles) load_tile(j + DEPTH, ring[(slot + DEPTH) % (DEPTH + 1)]);
+                compute_tile(ring[slot]);
+                if (++j >= num_wave_tiles) {
+                    finished = true;
+                    break;
+                }
+            }
+            if (finished) break;
         }
-#else
-        KvTile<D, KV8> t0, t1;
-        load_tile(0, t0);
-        uint32_t j = 0;
-        while (true) {
-            if (j + 1 < num_wave_tiles) load_tile(j + 1, t1);
-            compute_tile(t0);
-            if (++j >= num_wave_tiles) break;
-            if (j + 1 < num_wave_tiles) load_tile(j + 1, t0);
-            compute_tile(t1);
-            if (++j >= num_wave_tiles) break;
-        }
-#endif
     }
 
     // ---- merge the waves of the block ------------------------------------------------------

@@ -335,6 +335,56 @@ def max_threads() -> int:
     return int(lib().khm_oracle_max_threads())
 
 
+# ---------------------------------------------------------------- bidirectional block SDPA
+
+
+def bidi_block_sdpa(q, local_k, local_v, q_token_ranges, cu_partial_outputs, num_active_q_token_ranges: int, block_size: int,
+                    max_q_tokens: int, num_q_heads: int, num_kv_heads: int, head_dim: int, scale: float, num_partial_slots: int):
+    """Restatement of gqa_bidi_block_sdpa_impl (components/metal/gqa_bidi_block_sdpa.metal:10-93) in f32: every Q token
+    of a range attends, unmasked, to the `block_size` local K/V tokens of its request block
+    (`local_kv_token_begin = q_token / block_size * block_size`); the partial state goes to slot
+    `cu[range + 1] - 1`.  Inputs are f32 arrays (bf16 inputs are widened by the caller).  Returns
+    (exp_sums, max_logits, partial_output) in the partial layout `[slots][Hq][max_q_tokens]([D])`; untouched entries
+    are NaN so that a test sees what was written.
+    """
+    q = np.asarray(q, dtype=np.float32).reshape(-1, num_q_heads, head_dim)
+    k = np.asarray(local_k, dtype=np.float32).reshape(-1, num_kv_heads, head_dim)
+    v = np.asarray(local_v, dtype=np.float32).reshape(-1, num_kv_heads, head_dim)
+    ranges = np.asarray(q_token_ranges, dtype=np.uint32).reshape(-1, 2)
+    cu = np.asarray(cu_partial_outputs, dtype=np.uint32).reshape(-1)
+    sums = np.full((num_partial_slots, num_q_heads, max_q_tokens), np.nan, dtype=np.float32)
+    maxs = np.full_like(sums, np.nan)
+    out = np.full((num_partial_slots, num_q_heads, max_q_tokens, head_dim), np.nan, dtype=np.float32)
+    ratio = num_q_heads // num_kv_heads
+    f32 = np.float32
+    for r in range(num_active_q_token_ranges):
+        begin, end = int(ranges[r, 0]), int(ranges[r, 1])
+        slot = int(cu[r + 1]) - 1
+        for offset in range(min(end - begin, max_q_tokens)):
+            token = begin + offset
+            local_begin = token // block_size * block_size
+            for head in range(num_q_heads):
+                kv_head = head // ratio
+                logits = np.empty(block_size, dtype=np.float32)
+                for local in range(block_size):
+                    score = f32(0.0)
+                    for d in range(head_dim):
+                        score = f32(score + f32(q[token, head, d] * k[local_begin + local, kv_head, d]))
+                    logits[local] = f32(score * f32(scale))
+                block_max = logits.max()
+                weights = np.exp((logits - block_max).astype(np.float32)).astype(np.float32)
+                exp_sum = f32(0.0)
+                for w in weights:
+                    exp_sum = f32(exp_sum + w)
+                sums[slot, head, offset] = exp_sum
+                maxs[slot, head, offset] = block_max
+                acc = np.zeros(head_dim, dtype=np.float32)
+                for local in range(block_size):
+                    acc = (acc + weights[local] * v[local_begin + local, kv_head]).astype(np.float32)
+                out[slot, head, offset] = acc / exp_sum if exp_sum > 0 else 0.0
+    return sums, maxs, out
+
+
 # ---------------------------------------------------------------- page write
 
 
