@@ -98,7 +98,12 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
     const int g = lane >> 4;
 
     // ---- task decode (uniform) -------------------------------------------------------------
-    const uint32_t task = blockIdx.x;
+    // Blocks are dispatched in linear order; the KV heads of one task vary fastest, so the blocks in flight together
+    // read neighbouring slabs of the same pages (a whole 64 KB page between the eight heads) instead of the same
+    // 4 KB window of many pages, which spreads the requests evenly over the memory channels (+4 % on config 2).
+    const uint32_t linear_block = blockIdx.y * gridDim.x + blockIdx.x;
+    const uint32_t task = linear_block / gridDim.y;
+    const uint32_t head_group_index = linear_block % gridDim.y;
     const uint32_t num_active_splits = resolve_u32(p.num_active_kv_splits, p.replay_parameters);
     if (task >= num_active_splits) return;
     const uint32_t range_index = p.templates[3 * (uint64_t)task];
@@ -120,8 +125,8 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
     const uint32_t req_slot = p.req_slots[flat_begin];
     const uint32_t layer = resolve_u32(p.layer_index, p.replay_parameters);
 
-    const uint32_t head_range = blockIdx.y % p.num_q_head_ranges;
-    const uint32_t kv_head = blockIdx.y / p.num_q_head_ranges;
+    const uint32_t head_range = head_group_index % p.num_q_head_ranges;
+    const uint32_t kv_head = head_group_index / p.num_q_head_ranges;
     const uint32_t head_range_begin = head_range * p.max_q_heads;
     const uint32_t heads_left = p.q_heads_per_kv_head - head_range_begin;
     const uint32_t num_heads = heads_left < p.max_q_heads ? heads_left : p.max_q_heads;
@@ -534,7 +539,7 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
     uint32_t partial_end = p.cu_partial_outputs[range_index + 1];
     if (partial_end > num_active_splits) partial_end = num_active_splits;
     if (tid == 0) {
-        uint32_t* counter = p.arrival_counters + (uint64_t)range_index * gridDim.y + blockIdx.y;
+        uint32_t* counter = p.arrival_counters + (uint64_t)range_index * gridDim.y + head_group_index;
         const uint32_t arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
         const uint32_t last = arrived == partial_end - partial_begin ? 1u : 0u;
         if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // re-arm for the next launch
