@@ -380,6 +380,63 @@ def cpu_baseline(index: int = 2, seconds_hint: float = 20.0) -> dict:
     }
 
 
+def producer_rows(device, steps: int = 20) -> dict:
+    """The two kernels that feed the SDPA, at config 5's prefill shape (8 x 2048 new tokens, Hq=32 / Hkv=8, D=128): per-head
+    RMSNorm + RoPE of Q, and the K/V page write into FP8 pages.  Both are HBM bound; bytes are what the kernel must move."""
+    import torch
+
+    from khalamari_amd import kv_page_write, rms_norm_rope
+    from khalamari_amd._lib import ReplayU32
+
+    spec = CONFIGS[5]
+    hq, hkv, d = spec["hq"], spec["hkv"], spec["d"]
+    requests, new_tokens = 8, 2048
+    tokens = requests * new_tokens
+    generator = torch.Generator(device=device)
+    generator.manual_seed(77)
+
+    def timed(launch):
+        for _ in range(3):
+            launch()
+        torch.cuda.synchronize()
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for a, b in pairs:
+            a.record()
+            launch()
+            b.record()
+        torch.cuda.synchronize()
+        return float(np.mean([a.elapsed_time(b) for a, b in pairs])) * 1e3
+
+    result = {}
+    q = torch.randn((tokens, hq, d), device=device, dtype=torch.float32, generator=generator).to(torch.bfloat16)
+    q_out = torch.empty_like(q)
+    weight = torch.ones(d, device=device, dtype=torch.bfloat16)
+    positions = (torch.arange(tokens, device=device, dtype=torch.int32) % new_tokens).contiguous()
+    norm = rms_norm_rope.Compute(rms_norm_rope.Config.bf16(hq, d, d, 1e-6, 1_000_000.0))
+    us = timed(lambda: norm.invoke(rms_norm_rope.Shape(tokens), input=q, norm_weight=weight, flat_token_indices=positions, output=q_out,
+                                   num_active_tokens=ReplayU32.fixed(tokens)))
+    nbytes = 2 * q.numel() * 2
+    result["rms_norm_rope"] = {"workload": f"Q rows {tokens}x{hq}x{d} bf16, default RoPE", "kernel_us": us, "algorithmic_bytes": nbytes,
+                               "gbps": nbytes / us / 1e3, "roofline_frac": nbytes / us / 1e3 / HBM_PEAK_GBPS}
+
+    pages_per_request = new_tokens // TOKENS_PER_PAGE
+    page_bytes = 2 * hkv * TOKENS_PER_PAGE * d
+    layout = kv_page_write.PageTableLayout(requests, 1, pages_per_request, 1)
+    pages = torch.zeros(requests * pages_per_request * page_bytes, dtype=torch.uint8, device=device)
+    page_ids = torch.from_numpy(np.random.default_rng(3).permutation(requests * pages_per_request).astype(np.int32)).to(device)
+    flat_k = torch.randn((tokens, hkv, d), device=device, dtype=torch.float32, generator=generator).to(torch.bfloat16)
+    flat_v = torch.randn((tokens, hkv, d), device=device, dtype=torch.float32, generator=generator).to(torch.bfloat16)
+    req_slots = (torch.arange(tokens, device=device, dtype=torch.int32) // new_tokens).contiguous()
+    writer = kv_page_write.Compute(kv_page_write.Config(hkv, d, page_bytes))
+    shape = kv_page_write.Shape(tokens, layout)
+    us = timed(lambda: writer.invoke(shape, pages=pages, flat_k=flat_k, flat_v=flat_v, req_slots=req_slots, flat_token_indices=positions,
+                                     page_ids=page_ids, num_active_token_writes=ReplayU32.fixed(tokens), page_table_index=ReplayU32.fixed(0)))
+    nbytes = 2 * flat_k.numel() * 2 + 2 * flat_k.numel()
+    result["kv_page_write"] = {"workload": f"K/V rows {tokens}x{hkv}x{d} bf16 -> FP8 E4M3FN pages", "kernel_us": us, "algorithmic_bytes": nbytes,
+                               "gbps": nbytes / us / 1e3, "roofline_frac": nbytes / us / 1e3 / HBM_PEAK_GBPS}
+    return result
+
+
 def _cpu_model() -> str:
     try:
         with open("/proc/cpuinfo") as handle:
@@ -453,6 +510,10 @@ def main() -> int:
                 torch.cuda.empty_cache()
             except Exception as error:
                 others[f"config{index}_fp8_pages"] = {"workload": CONFIGS[index]["name"] + " [FP8 E4M3FN pages]", "error": str(error)}
+        try:
+            others["producers"] = producer_rows(device)
+        except Exception as error:
+            others["producers"] = {"error": str(error)}
     prefill = head["bound"] == "mfma"
     line = {
         "metric": "paged GQA prefill bf16 MFMA TFLOP/s" if prefill else "paged GQA decode achieved HBM GB/s (split-KV Map + LSE Reduce per step)",

@@ -406,6 +406,50 @@ int khm_bidi_block_sdpa(const khm_bidi_block_sdpa_config* config, const khm_bidi
                         const uint32_t* replay_parameters, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Per-head RMSNorm + rotary embedding: components/rms_norm_rope.rs:53-403, metal/rms_norm_rope.metal:6-174
+ * The step that produces the SDPA's Q (and K before the page write): out = rope(weight * x * rsqrt(mean(x^2) + eps)).
+ * ------------------------------------------------------------------------------------------ */
+typedef enum khm_rope_scaling_kind { KHM_ROPE_SCALING_DEFAULT = 0, KHM_ROPE_SCALING_YARN = 1 } khm_rope_scaling_kind;
+/* rms_norm_rope::RopeScaling (rms_norm_rope.rs:53-64); the Yarn fields are ignored for the default kind. */
+typedef struct khm_rope_scaling {
+    uint32_t kind;
+    float factor;
+    float attention_factor;
+    float beta_fast;
+    float beta_slow;
+    uint32_t original_max_position_embeddings;
+    uint32_t truncate; /* 0 / 1 */
+} khm_rope_scaling;
+/* rms_norm_rope::Config (rms_norm_rope.rs:77-87). */
+typedef struct khm_rms_norm_rope_config {
+    uint32_t num_heads;
+    uint32_t head_dim;
+    uint32_t rope_dim;
+    float eps;
+    float rope_theta;
+    khm_rope_scaling rope_scaling;
+    uint32_t dtype;             /* input/output: KHM_DTYPE_F32 or KHM_DTYPE_BF16 */
+    uint32_t norm_weight_dtype; /* KHM_DTYPE_F32 or KHM_DTYPE_BF16 */
+} khm_rms_norm_rope_config;
+/* rms_norm_rope::Buffers (rms_norm_rope.rs:286-292): input/output [T][num_heads][head_dim], norm_weight [head_dim],
+ * flat_token_indices u32 [T] (the rotary positions). */
+typedef struct khm_rms_norm_rope_buffers {
+    khm_buffer input;
+    khm_buffer norm_weight;
+    khm_buffer flat_token_indices;
+    khm_buffer output;
+} khm_rms_norm_rope_buffers;
+/* RopeScaling::yarn_kernel_parameters (rms_norm_rope.rs:206-243): the Yarn correction range (host only). */
+int khm_rms_norm_rope_yarn_correction_range(const khm_rms_norm_rope_config* config, float* low, float* high);
+/* RopeScaling::kernel_parameters (rms_norm_rope.rs:245-270): rope_dim / 2 inverse frequencies and the attention
+ * factor (host only). */
+int khm_rms_norm_rope_kernel_parameters(const khm_rms_norm_rope_config* config, float* inverse_frequencies, uint32_t capacity,
+                                        float* attention_factor);
+/* Compute::invoke + Invocation::record (rms_norm_rope.rs:312-384): one launch, enqueued on `stream`. */
+int khm_rms_norm_rope(const khm_rms_norm_rope_config* config, uint32_t num_total_tokens, const khm_rms_norm_rope_buffers* buffers,
+                      khm_replay_u32 num_active_tokens, const uint32_t* replay_parameters, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Executor-side host logic that feeds the component (CPU only, no HIP calls)
  * ------------------------------------------------------------------------------------------ */
 

@@ -199,6 +199,24 @@ class BidiBlockSdpaBuffers(ctypes.Structure):
                 ("partial_exp_sums", Buffer), ("partial_max_logits", Buffer), ("partial_output", Buffer)]
 
 
+class RopeScalingStruct(ctypes.Structure):
+    """`rms_norm_rope::RopeScaling`; kind 0 = default, 1 = Yarn."""
+
+    _fields_ = [("kind", u32), ("factor", ctypes.c_float), ("attention_factor", ctypes.c_float), ("beta_fast", ctypes.c_float),
+                ("beta_slow", ctypes.c_float), ("original_max_position_embeddings", u32), ("truncate", u32)]
+
+
+class RmsNormRopeConfig(ctypes.Structure):
+    """`rms_norm_rope::Config`."""
+
+    _fields_ = [("num_heads", u32), ("head_dim", u32), ("rope_dim", u32), ("eps", ctypes.c_float), ("rope_theta", ctypes.c_float),
+                ("rope_scaling", RopeScalingStruct), ("dtype", u32), ("norm_weight_dtype", u32)]
+
+
+class RmsNormRopeBuffers(ctypes.Structure):
+    _fields_ = [("input", Buffer), ("norm_weight", Buffer), ("flat_token_indices", Buffer), ("output", Buffer)]
+
+
 # Every symbol `include/khm_gqa_sdpa.h` declares; checked by tests/test_abi.py.
 EXPORTED_SYMBOLS = (
     "khm_last_error", "khm_version",
@@ -216,6 +234,7 @@ EXPORTED_SYMBOLS = (
     "khm_fp8_e4m3_to_bf16_device", "khm_bf16_to_fp8_e4m3_device",
     "khm_kv_page_write_num_tokens_per_page", "khm_kv_page_write",
     "khm_bidi_block_sdpa",
+    "khm_rms_norm_rope_yarn_correction_range", "khm_rms_norm_rope_kernel_parameters", "khm_rms_norm_rope",
     "khm_replay_bucket_policy_create", "khm_replay_bucket_policy_destroy", "khm_replay_bucket_policy_max_capacity",
     "khm_replay_bucket_policy_buckets", "khm_replay_bucket_policy_capacity", "khm_replay_bucket_policy_capacity_allow_zero",
     "khm_request_shapes_from_batch",
@@ -297,6 +316,11 @@ def lib() -> ctypes.CDLL:
                                          ctypes.POINTER(KvPageWriteBuffers), ReplayU32, ReplayU32, ctypes.c_void_p, ctypes.c_void_p]
     handle.khm_bidi_block_sdpa.argtypes = [ctypes.POINTER(BidiBlockSdpaConfig), ctypes.POINTER(BidiBlockSdpaShape),
                                            ctypes.POINTER(BidiBlockSdpaBuffers), ReplayU32, ctypes.c_void_p, ctypes.c_void_p]
+    float_p = ctypes.POINTER(ctypes.c_float)
+    handle.khm_rms_norm_rope_yarn_correction_range.argtypes = [ctypes.POINTER(RmsNormRopeConfig), float_p, float_p]
+    handle.khm_rms_norm_rope_kernel_parameters.argtypes = [ctypes.POINTER(RmsNormRopeConfig), float_p, u32, float_p]
+    handle.khm_rms_norm_rope.argtypes = [ctypes.POINTER(RmsNormRopeConfig), u32, ctypes.POINTER(RmsNormRopeBuffers), ReplayU32,
+                                         ctypes.c_void_p, ctypes.c_void_p]
     _lib = handle
     return handle
 

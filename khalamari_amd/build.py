@@ -24,6 +24,7 @@ SOURCES = [
     "components.hip",
     "kv_page_write.hip",
     "bidi_block_sdpa.hip",
+    "rms_norm_rope.hip",
 ]
 
 HIPCC_FLAGS = [

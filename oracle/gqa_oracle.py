@@ -335,6 +335,81 @@ def max_threads() -> int:
     return int(lib().khm_oracle_max_threads())
 
 
+# ---------------------------------------------------------------- per-head RMSNorm + rotary embedding
+
+
+def yarn_correction_range(rope_dim: int, rope_theta: float, beta_fast: float, beta_slow: float, original_max_position_embeddings: int,
+                          truncate: bool):
+    """`RopeScaling::yarn_kernel_parameters` (components/rms_norm_rope.rs:206-243): the (low, high) rotary-pair range over
+    which Yarn ramps from the unscaled to the interpolated frequency.  f64 inside the logarithms, f32 results."""
+    def correction(rotations):
+        value = rope_dim * np.log(np.float64(original_max_position_embeddings) / (np.float64(np.float32(rotations)) * 2.0 * np.pi))
+        return np.float32(value / (2.0 * np.log(np.float64(np.float32(rope_theta)))))
+
+    low = max(correction(beta_fast), np.float32(0.0))
+    high = min(correction(beta_slow), np.float32(max(rope_dim - 1, 0)))
+    if truncate:
+        low, high = np.floor(low), np.ceil(high)
+    if not low <= high:
+        raise ValueError("Yarn correction range must be ordered")
+    if low == high:
+        high = np.float32(high + np.float32(0.001))
+    return np.float32(low), np.float32(high)
+
+
+def rope_kernel_parameters(rope_dim: int, rope_theta: float, yarn=None):
+    """`RopeScaling::kernel_parameters` (rms_norm_rope.rs:245-270): (inverse_frequencies f32[rope_dim/2], attention_factor).
+    `yarn` is None or a dict with factor, attention_factor, beta_fast, beta_slow, original_max_position_embeddings, truncate."""
+    rope_half = rope_dim // 2
+    dims = np.arange(rope_half, dtype=np.float32)
+    # powf(theta, -(d / half)) with f32 operands, correctly rounded (f64 power, then one rounding), as a libm powf returns;
+    # numpy's own f32 power is an ulp off for some pairs, and at position 2^18 one ulp of a frequency moves the output by 1e-2
+    inverse = np.power(np.float64(np.float32(rope_theta)), -(dims / np.float32(rope_half)).astype(np.float64)).astype(np.float32)
+    if yarn is None:
+        return inverse, np.float32(1.0)
+    low, high = yarn_correction_range(rope_dim, rope_theta, yarn["beta_fast"], yarn["beta_slow"], yarn["original_max_position_embeddings"],
+                                      yarn["truncate"])
+    ramp = np.clip((dims - low) / (high - low), np.float32(0.0), np.float32(1.0)).astype(np.float32)
+    scale = np.float32(1.0) + ramp * (np.float32(1.0) / np.float32(yarn["factor"]) - np.float32(1.0))
+    return (inverse * scale).astype(np.float32), np.float32(yarn["attention_factor"])
+
+
+def rms_norm_rope(input_values, norm_weight, positions, num_heads: int, head_dim: int, rope_dim: int, eps: float, rope_theta: float,
+                  yarn=None, io_bf16: bool = False, weight_bf16: bool = False) -> np.ndarray:
+    """`rms_norm_rope_impl` (components/metal/rms_norm_rope.metal:22-120) for rows [T][num_heads][head_dim].
+
+    `input_values` / the result are f32 values, or bf16 bit patterns (uint16) when `io_bf16`; `norm_weight` likewise under
+    `weight_bf16`.  With bf16 input AND bf16 weight the normalized value and its product with the weight are each
+    rounded to bf16 (apply_norm, rms_norm_rope.metal:14-16); every other combination multiplies in f32.  The square sum
+    runs over the row in index order in f32."""
+    x = bf16_bits_to_f32(input_values) if io_bf16 else np.asarray(input_values, dtype=np.float32)
+    w = bf16_bits_to_f32(norm_weight) if weight_bf16 else np.asarray(norm_weight, dtype=np.float32)
+    x = x.reshape(-1, num_heads, head_dim)
+    positions = np.asarray(positions, dtype=np.uint32)
+    inverse, attention_factor = rope_kernel_parameters(rope_dim, rope_theta, yarn)
+    rope_half = rope_dim // 2
+    out = np.zeros_like(x)
+    for token in range(x.shape[0]):
+        theta = (np.float32(positions[token]) * inverse).astype(np.float32)
+        # the rotation angle is an f32; its sine and cosine are evaluated in f64 and rounded
+        cos, sin = np.cos(theta.astype(np.float64)).astype(np.float32), np.sin(theta.astype(np.float64)).astype(np.float32)
+        for head in range(num_heads):
+            row = x[token, head]
+            acc = np.float32(0.0)
+            for value in row:
+                acc = np.float32(acc + value * value)
+            inv_rms = np.float32(1.0) / np.sqrt(np.float32(acc / np.float32(head_dim) + np.float32(eps)), dtype=np.float32)
+            if io_bf16 and weight_bf16:
+                normed = bf16_round(w * bf16_round(row * inv_rms))
+            else:
+                normed = (w * row * inv_rms).astype(np.float32)
+            first, second = normed[:rope_half], normed[rope_half:rope_dim]
+            out[token, head, :rope_half] = attention_factor * (first * cos - second * sin)
+            out[token, head, rope_half:rope_dim] = attention_factor * (first * sin + second * cos)
+            out[token, head, rope_dim:] = normed[rope_dim:]
+    return f32_to_bf16_bits(out) if io_bf16 else out
+
+
 # ---------------------------------------------------------------- bidirectional block SDPA
 
 
