@@ -13,6 +13,13 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef short s16x4v __attribute__((ext_vector_type(4)));
+
+// LDS transpose read: lane r of every 16-lane group passes the address of 4 consecutive bf16; lane i receives
+// element (i % 4) of the rows given by lanes i/4, i/4 + 4, i/4 + 8, i/4 + 12 of its group.
+__device__ __forceinline__ s16x4v lds_read_tr16(const unsigned char* address) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4v __attribute__((address_space(3)))*)(address));
+}
 
 __device__ __forceinline__ uint32_t resolve_u32(DeviceReplayU32 r, const uint32_t* params) {
     return r.is_parameter ? params[r.value] : r.value;

@@ -49,7 +49,7 @@ struct KvTile {
 
 template <int D, int NT, int NWAVES>
 struct MapSmem {
-    static constexpr int kVRowBytes = D * 2 + 8;           // +8 B: conflict-free transposed reads
+    static constexpr int kVRowBytes = D * 2 + 32;          // +32 B: rows 8 banks apart, conflict-free transposed reads
     static constexpr int kVBytes = NWAVES * 16 * kVRowBytes;
     static constexpr int kCols = NT * 16;
     static constexpr int kORowFloats = D + 4;
@@ -57,7 +57,7 @@ struct MapSmem {
     static constexpr int kUnionBytes = kVBytes > kOBytes ? kVBytes : kOBytes;
     static constexpr int kQRowBytes = D * 2 + 16;
     static constexpr int kQBytes = kCols * kQRowBytes;
-    static constexpr int kStatsBytes = (NWAVES + 1) * kCols * 2 * 4;
+    static constexpr int kStatsBytes = (NWAVES + 1) * kCols * 3 * 4;   // (reference, sum, maximum) per wave and column
     static constexpr int kTotal = kUnionBytes + kQBytes + kStatsBytes;
 };
 
@@ -281,15 +281,21 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
 
     // ---- online-softmax state --------------------------------------------------------------
     f32x4 acc[NT][MT];
-    float run_max[NT], run_sum[NT];
+    // Weights are exp2(score - ref) for a per-column reference that only moves when a score exceeds it by more than
+    // kRescaleThreshold (so weights stay below 2^8 and the accumulator is rescaled a few times per block, not per
+    // tile); lane_top is the lane's own largest score relative to ref, run_sum the lane's own part of the column sum.
+    constexpr float kRescaleThreshold = 8.0f;
+    float ref[NT], lane_top[NT], run_sum[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        run_max[nt] = -INFINITY;
+        ref[nt] = 0.0f;
+        lane_top[nt] = -INFINITY;
         run_sum[nt] = 0.0f;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     }
     unsigned char* v_lds = v_lds_all + wave * 16 * Smem::kVRowBytes;
+    const unsigned char* v_transposed = v_lds + (g * 4 + (r16 >> 2)) * Smem::kVRowBytes + (r16 & 3) * 8;
 
     auto compute_tile = [&](const KvTile<D, KV8>& tile) {
         const uint32_t first_token = tile.first_token;
@@ -322,36 +328,57 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
         // Softmax weights go into the second MFMA as hi + lo bf16 pairs (p = hi + lo to ~2^-17): this kernel is
         // bandwidth-bound, so the second product is free and the weights keep f32-like accuracy as in the reference.
         uint32_t p_bits[NT][2], p_low[NT][2];
+        float v[NT][4], tile_top[NT];
+        bool lane_wants_move = false;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-            float v[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) v[i] = s[nt][i] * p.scale_log2e;
+            for (int i = 0; i < 4; ++i) v[nt][i] = __builtin_fmaf(s[nt][i], p.scale_log2e, -ref[nt]);
             if (!interior) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const uint32_t token = first_token + g * 4 + i;
-                    v[i] = (token >= col_lo[nt] && token < col_hi[nt]) ? v[i] : -INFINITY;
+                    v[nt][i] = (token >= col_lo[nt] && token < col_hi[nt]) ? v[nt][i] : -INFINITY;
                 }
             }
-            float tile_max = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
-            tile_max = max_over_rows(tile_max);
-            const float next_max = fmaxf(run_max[nt], tile_max);
-            const float safe_max = next_max == -INFINITY ? 0.0f : next_max;
-            const float alpha = fast_exp2(run_max[nt] - safe_max);
-            run_max[nt] = next_max;
+            tile_top[nt] = fmaxf(fmaxf(v[nt][0], v[nt][1]), fmaxf(v[nt][2], v[nt][3]));
+            // a lane that has not seen a visible key yet cannot know whether its column has a reference
+            lane_wants_move = lane_wants_move | (tile_top[nt] > kRescaleThreshold) | (lane_top[nt] == -INFINITY);
+        }
+        if (__builtin_amdgcn_ballot_w64(lane_wants_move) != 0) {
+            // rare: the four lanes of a column agree on its maximum, move the reference, rescale what was accumulated
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const float column_top = max_over_rows(tile_top[nt]);
+                const float column_seen = max_over_rows(lane_top[nt]);
+                const bool first = column_seen == -INFINITY;
+                const bool move = column_top > kRescaleThreshold || (first && column_top > -INFINITY);
+                const float shift = move ? column_top : 0.0f;
+                const float alpha = first ? 0.0f : fast_exp2(-shift);   // nothing is accumulated before the first key
+                ref[nt] += shift;
+                lane_top[nt] -= shift;
+                tile_top[nt] -= shift;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v[nt][i] -= shift;
+                run_sum[nt] *= alpha;
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    asm volatile("" : "+a"(acc[nt][mt]));   // the move out of the AGPRs belongs to this branch
+                    acc[nt][mt] *= alpha;
+                }
+            }
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            lane_top[nt] = fmaxf(lane_top[nt], tile_top[nt]);
             float e[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) e[i] = fast_exp2(v[i] - safe_max);
-            run_sum[nt] = run_sum[nt] * alpha + ((e[0] + e[1]) + (e[2] + e[3]));
+            for (int i = 0; i < 4; ++i) e[i] = fast_exp2(v[nt][i]);
+            run_sum[nt] += (e[0] + e[1]) + (e[2] + e[3]);
             p_bits[nt][0] = pack_bf16x2(e[0], e[1]);
             p_bits[nt][1] = pack_bf16x2(e[2], e[3]);
             p_low[nt][0] = pack_bf16x2(e[0] - bf16_bits_to_f32(p_bits[nt][0] & 0xffffu), e[1] - bf16_bits_to_f32(p_bits[nt][0] >> 16));
             p_low[nt][1] = pack_bf16x2(e[2] - bf16_bits_to_f32(p_bits[nt][1] & 0xffffu), e[3] - bf16_bits_to_f32(p_bits[nt][1] >> 16));
-            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) acc[nt][mt] *= alpha;
-            }
         }
         // V tile -> wave-private LDS (rows outside the block's KV range are zeroed: an unused
         // page slot may hold anything, and 0 * NaN would poison the accumulator).
@@ -359,27 +386,27 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
             const uint32_t row_in_load = lane / LANES_PER_ROW;
             const uint32_t chunk_in_row = lane % LANES_PER_ROW;
             const bool edge = first_token < blk_lo || first_token + 16 > blk_hi;
-#pragma unroll
-            for (int i = 0; i < LOADS; ++i) {
+            auto stage = [&](int i, uint4 value) __attribute__((always_inline)) {
                 const uint32_t row = i * ROWS_PER_LOAD + row_in_load;
-                uint4 value = tile.v[i];
-                if (edge) {
-                    const uint32_t token = first_token + row;
-                    if (token < blk_lo || token >= blk_hi) value = make_uint4(0, 0, 0, 0);
-                }
                 if constexpr (KV8) {
                     // sixteen codes -> sixteen bf16: the staged tile is bf16 whatever the page format
                     const uint4 low = fp8x8_to_bf16x8(make_uint2(value.x, value.y));
                     const uint4 high = fp8x8_to_bf16x8(make_uint2(value.z, value.w));
-                    uint2* target = reinterpret_cast<uint2*>(v_lds + row * Smem::kVRowBytes + chunk_in_row * 32);
-                    target[0] = make_uint2(low.x, low.y);
-                    target[1] = make_uint2(low.z, low.w);
-                    target[2] = make_uint2(high.x, high.y);
-                    target[3] = make_uint2(high.z, high.w);
+                    uint4* target = reinterpret_cast<uint4*>(v_lds + row * Smem::kVRowBytes + chunk_in_row * 32);
+                    target[0] = low;
+                    target[1] = high;
                 } else {
-                    uint2* target = reinterpret_cast<uint2*>(v_lds + row * Smem::kVRowBytes + chunk_in_row * 16);
-                    target[0] = make_uint2(value.x, value.y);
-                    target[1] = make_uint2(value.z, value.w);
+                    *reinterpret_cast<uint4*>(v_lds + row * Smem::kVRowBytes + chunk_in_row * 16) = value;
+                }
+            };
+            if (!edge) {
+#pragma unroll
+                for (int i = 0; i < LOADS; ++i) stage(i, tile.v[i]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < LOADS; ++i) {
+                    const uint32_t token = first_token + i * ROWS_PER_LOAD + row_in_load;
+                    stage(i, (token < blk_lo || token >= blk_hi) ? make_uint4(0, 0, 0, 0) : tile.v[i]);
                 }
             }
         }
@@ -387,14 +414,11 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         // O^T += V^T . P^T
+        // ds_read_b64_tr_b16: the lane passes (row 4g + r/4, dims mt*16 + 4*(r%4) .. +3) and receives dim mt*16 + r of
+        // rows 4g .. 4g+3, which is the A fragment of V^T.
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            const unsigned char* column = v_lds + (g * 4) * Smem::kVRowBytes + (mt * 16 + r16) * 2;
-            s16x4 a;
-            a[0] = *reinterpret_cast<const short*>(column);
-            a[1] = *reinterpret_cast<const short*>(column + Smem::kVRowBytes);
-            a[2] = *reinterpret_cast<const short*>(column + 2 * Smem::kVRowBytes);
-            a[3] = *reinterpret_cast<const short*>(column + 3 * Smem::kVRowBytes);
+            const s16x4 a = __builtin_bit_cast(s16x4, lds_read_tr16(v_transposed + mt * 32));
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const uint2 b_bits = make_uint2(p_bits[nt][0], p_bits[nt][1]);
@@ -405,6 +429,12 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
+        // The accumulator stays in the AGPR half of the register file from tile to tile (only the rare rescale moves
+        // it through VGPRs); without the pin the compiler keeps a second copy in VGPRs and refreshes it after every tile.
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) asm volatile("" : "+a"(acc[nt][mt]));
     };
 
     // ---- main loop: a ring of register buffers, loads DEPTH tiles ahead ----------------------
@@ -433,33 +463,42 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
     }
 
     // ---- merge the waves of the block ------------------------------------------------------
+    float wave_ref[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         run_sum[nt] = sum_over_rows(run_sum[nt]);
+        const float top = max_over_rows(lane_top[nt]);
+        wave_ref[nt] = top == -INFINITY ? -INFINITY : ref[nt];     // a wave that saw no visible key has no reference
         if (g == 0) {
-            stats_lds[(wave * COLS + nt * 16 + r16) * 2] = run_max[nt];
-            stats_lds[(wave * COLS + nt * 16 + r16) * 2 + 1] = run_sum[nt];
+            float* stats = stats_lds + (wave * COLS + nt * 16 + r16) * 3;
+            stats[0] = wave_ref[nt];
+            stats[1] = run_sum[nt];
+            stats[2] = top == -INFINITY ? -INFINITY : ref[nt] + top;   // the wave's true maximum
         }
     }
     __syncthreads();  // also: every wave is done with its V staging tile
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         const int c = nt * 16 + r16;
-        float global_max = -INFINITY;
+        float global_ref = -INFINITY, global_max = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < NWAVES; ++w) global_max = fmaxf(global_max, stats_lds[(w * COLS + c) * 2]);
+        for (int w = 0; w < NWAVES; ++w) {
+            global_ref = fmaxf(global_ref, stats_lds[(w * COLS + c) * 3]);
+            global_max = fmaxf(global_max, stats_lds[(w * COLS + c) * 3 + 2]);
+        }
         float global_sum = 0.0f;
 #pragma unroll
         for (int w = 0; w < NWAVES; ++w) {
-            const float wave_sum = stats_lds[(w * COLS + c) * 2 + 1];
-            if (wave_sum > 0.0f) global_sum += wave_sum * fast_exp2(stats_lds[(w * COLS + c) * 2] - global_max);
+            const float wave_sum = stats_lds[(w * COLS + c) * 3 + 1];
+            if (wave_sum > 0.0f) global_sum += wave_sum * fast_exp2(stats_lds[(w * COLS + c) * 3] - global_ref);
         }
-        const float own = (run_sum[nt] > 0.0f && global_sum > 0.0f) ? fast_exp2(run_max[nt] - global_max) / global_sum : 0.0f;
+        const float own = (run_sum[nt] > 0.0f && global_sum > 0.0f) ? fast_exp2(wave_ref[nt] - global_ref) / global_sum : 0.0f;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[nt][mt] *= own;
         if (wave == 0 && g == 0) {
-            stats_lds[(NWAVES * COLS + c) * 2] = global_sum > 0.0f ? global_max * 0.6931471805599453f : -INFINITY;
-            stats_lds[(NWAVES * COLS + c) * 2 + 1] = global_sum;
+            // published relative to the true maximum, as the partial-state contract says
+            stats_lds[(NWAVES * COLS + c) * 3] = global_sum > 0.0f ? global_max * 0.6931471805599453f : -INFINITY;
+            stats_lds[(NWAVES * COLS + c) * 3 + 1] = global_sum > 0.0f ? global_sum * fast_exp2(global_ref - global_max) : 0.0f;
         }
     }
     for (int w = 0; w < NWAVES; ++w) {
@@ -520,11 +559,11 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
         if (token_offset < num_q && local_head < num_heads) {
             const uint64_t state = ((uint64_t)task * p.num_q_heads + first_q_head + local_head) * p.max_q_tokens + token_offset;
             if (fused) {
-                coherent_store_f32(p.max_logits + state, stats_lds[(NWAVES * COLS + c) * 2]);
-                coherent_store_f32(p.exp_sums + state, stats_lds[(NWAVES * COLS + c) * 2 + 1]);
+                coherent_store_f32(p.max_logits + state, stats_lds[(NWAVES * COLS + c) * 3]);
+                coherent_store_f32(p.exp_sums + state, stats_lds[(NWAVES * COLS + c) * 3 + 1]);
             } else {
-                p.max_logits[state] = stats_lds[(NWAVES * COLS + c) * 2];
-                p.exp_sums[state] = stats_lds[(NWAVES * COLS + c) * 2 + 1];
+                p.max_logits[state] = stats_lds[(NWAVES * COLS + c) * 3];
+                p.exp_sums[state] = stats_lds[(NWAVES * COLS + c) * 3 + 1];
             }
         }
     }

@@ -33,8 +33,6 @@
 #endif
 namespace khm {
 
-typedef short s16x4v __attribute__((ext_vector_type(4)));
-
 template <int D, int BK, int NSTAGES>
 struct TileSmem {
     static constexpr int kRowBytes = D * 2;
@@ -42,11 +40,6 @@ struct TileSmem {
     static constexpr int kBytes = 2 /*K,V*/ * NSTAGES * kTileBytes;
 };
 
-// LDS transpose read: lane r of every 16-lane group passes the address of 4 consecutive bf16; lane i receives
-// element (i % 4) of the rows given by lanes i/4, i/4 + 4, i/4 + 8, i/4 + 12 of its group.
-__device__ __forceinline__ s16x4v lds_read_tr16(const unsigned char* address) {
-    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4v __attribute__((address_space(3)))*)(address));
-}
 
 // 16 bytes per lane from global memory to LDS: lane l of the wave reads uniform_base + lane_offset and lands at
 // lds_address + 16 * l (lds_address is wave-uniform and travels in M0).  Written as inline assembly on purpose: the
