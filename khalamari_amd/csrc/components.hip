@@ -89,6 +89,29 @@ static ReduceKernel select_reduce_kernel(uint32_t head_dim, bool ranged) {
     return nullptr;
 }
 
+// Rows with few partials merge faster one row per thread group (no LDS pass); the shape's average decides.
+constexpr uint32_t kFewPartialsPerRow = 16;
+
+static ReduceKernel select_reduce_rows_kernel(uint32_t head_dim, bool ranged) {
+    if (head_dim == 128) return ranged ? split_kv_reduce_rows_kernel<128, true> : split_kv_reduce_rows_kernel<128, false>;
+    if (head_dim == 256) return ranged ? split_kv_reduce_rows_kernel<256, true> : split_kv_reduce_rows_kernel<256, false>;
+    return nullptr;
+}
+
+// Launches the Reduce over `units` tokens (flat) or Q ranges (ranged) of `max_q_tokens` token slots each.
+static void launch_reduce_kernel(const khm_gqa_sdpa_config& config, const khm_gqa_sdpa_shape& shape, bool ranged, uint32_t units,
+                                 uint32_t max_q_tokens, ReduceKernel sliced, const ReduceParams& p, hipStream_t stream) {
+    const bool few = (uint64_t)shape.num_total_sdpa_map_task_templates <= (uint64_t)kFewPartialsPerRow * units;
+    if (few) {
+        const uint64_t rows = (uint64_t)units * max_q_tokens * config.num_q_heads;
+        const uint32_t rows_per_block = kReduceThreads / (config.head_dim / 4);
+        hipLaunchKernelGGL(select_reduce_rows_kernel(config.head_dim, ranged), dim3((uint32_t)((rows + rows_per_block - 1) / rows_per_block)),
+                           dim3(kReduceThreads), 0, stream, p);
+    } else {
+        hipLaunchKernelGGL(sliced, dim3(units * max_q_tokens, config.num_q_heads, 1), dim3(kReduceThreads), 0, stream, p);
+    }
+}
+
 static DeviceReplayU32 to_device(khm_replay_u32 value) { return DeviceReplayU32{value.is_parameter, value.value}; }
 
 // ReplayU32::validate_range for Fixed values; Parameters are range-checked by whoever fills the block
@@ -401,8 +424,7 @@ static int launch_sliced_kv_reduce(const khm_sliced_kv* compute, const khm_slice
     p.head_dim = config.head_dim;
     p.max_q_tokens = 1;
     p.partial_is_f32 = config.partial_dtype == KHM_DTYPE_F32;
-    const dim3 grid(shape.num_total_tokens, config.num_q_heads, 1);
-    hipLaunchKernelGGL(compute->reduce, grid, dim3(kReduceThreads), 0, static_cast<hipStream_t>(stream), p);
+    launch_reduce_kernel(config, shape, false, shape.num_total_tokens, 1, compute->reduce, p, static_cast<hipStream_t>(stream));
     return check_launch("sliced-KV reduce");
 }
 
@@ -642,8 +664,8 @@ extern "C" int khm_sliced_q_reduce(const khm_sliced_q* compute, const khm_sliced
     p.partial_is_f32 = config.partial_dtype == KHM_DTYPE_F32;
     KHM_REQUIRE(!mul_overflows_u32(shape.num_total_q_token_tiles, compute->variant.map_max_q_tokens),
                 "GQA SplitKV SlicedQ reduce grid exceeds the u32 domain");
-    const dim3 grid(shape.num_total_q_token_tiles * compute->variant.map_max_q_tokens, config.num_q_heads, 1);
-    hipLaunchKernelGGL(compute->reduce, grid, dim3(kReduceThreads), 0, static_cast<hipStream_t>(stream), p);
+    launch_reduce_kernel(config, shape, true, shape.num_total_q_token_tiles, compute->variant.map_max_q_tokens, compute->reduce, p,
+                         static_cast<hipStream_t>(stream));
     return check_launch("sliced-Q reduce");
 }
 

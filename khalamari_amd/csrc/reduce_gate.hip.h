@@ -72,6 +72,39 @@ __global__ __launch_bounds__(kReduceThreads) void split_kv_reduce_kernel(const R
     }
 }
 
+// The same merge for rows with few partials (speculative-verify tiles have about ten): a group of D/4 threads owns one
+// (token, head) row and walks all of its partials itself, eight loads in flight, so a block serves 256 / (D/4) rows
+// and nothing passes through LDS.  Rows are numbered (unit * max_q_tokens + token slot) * num_q_heads + head.
+template <int D, bool RANGED>
+__global__ __launch_bounds__(kReduceThreads) void split_kv_reduce_rows_kernel(const ReduceParams p) {
+    constexpr int CHUNKS = D / 4;
+    constexpr int ROWS = kReduceThreads / CHUNKS;
+    const int chunk = threadIdx.x % CHUNKS;
+    const uint64_t row = (uint64_t)blockIdx.x * ROWS + threadIdx.x / CHUNKS;
+    const uint32_t max_q = RANGED ? p.max_q_tokens : 1u;
+    const uint64_t slot = row / p.num_q_heads;
+    const uint32_t head = (uint32_t)(row - slot * p.num_q_heads);
+    const uint32_t unit = (uint32_t)(slot / max_q);
+    const uint32_t local = (uint32_t)(slot - (uint64_t)unit * max_q);
+    if (unit >= resolve_u32(p.num_active, p.replay_parameters)) return;
+    uint32_t flat_begin = unit, num_q = 1;
+    if (RANGED) {
+        flat_begin = p.q_token_ranges[2 * (uint64_t)unit];
+        num_q = p.q_token_ranges[2 * (uint64_t)unit + 1] - flat_begin;
+        if (num_q > max_q) num_q = max_q;
+    }
+    if (local >= num_q) return;
+    const uint32_t begin = p.cu_partial_outputs[unit];
+    const uint32_t end = p.cu_partial_outputs[unit + 1];
+    MergeState state = merge_state_empty();
+    if (end > begin) {
+        merge_partial_slice<D, false>(state, p.max_logits, p.exp_sums, p.partial, p.partial_is_f32 != 0, begin, end, 1, begin, p.num_q_heads, head,
+                                      max_q, local, chunk);
+    }
+    const uint64_t out_index = ((uint64_t)(flat_begin + local) * p.num_q_heads + head) * D + chunk * 4;
+    merge_store_output(state, p.output, p.gates, out_index);
+}
+
 // gqa_activation_gate_{f32,bf16} (gqa_activation_gate.metal:28-59): one thread per element.
 __global__ __launch_bounds__(256) void activation_gate_kernel(const GateParams p) {
     const uint64_t total = (uint64_t)resolve_u32(p.num_active_tokens, p.replay_parameters) * p.values_per_token;
