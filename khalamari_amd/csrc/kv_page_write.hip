@@ -34,17 +34,17 @@ struct PageWriteParams {
     uint32_t num_page_ids_per_block;
 };
 
-// One thread moves eight consecutive dims of one (write, KV head) row, for K and for V: a 16-byte load each, then a
-// 16-byte (bf16 pages) or 8-byte (FP8 pages) store each.  Head dims that are no multiple of eight take the scalar tail.
+// A block serves one token write (blockIdx.x), so the request slot, the page-table walk and the page address are
+// wave-uniform scalar work; a thread moves eight consecutive dims of one KV head's row, for K and for V: a 16-byte load
+// each, then a 16-byte (bf16 pages) or 8-byte (FP8 pages) store each.  Head dims that are no multiple of eight take the
+// scalar tail.
 template <bool FP8_PAGES>
-__global__ __launch_bounds__(256) void kv_page_write_kernel(const PageWriteParams p) {
+__global__ __launch_bounds__(1024) void kv_page_write_kernel(const PageWriteParams p) {
+    const uint32_t write_index = blockIdx.x;
+    if (write_index >= resolve_u32(p.num_active_token_writes, p.replay_parameters)) return;
     const uint32_t chunks_per_row = (p.head_dim + 7) / 8;
-    const uint64_t chunks_per_write = (uint64_t)p.num_kv_heads * chunks_per_row;
-    const uint64_t total = (uint64_t)resolve_u32(p.num_active_token_writes, p.replay_parameters) * chunks_per_write;
-    const uint64_t gid = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-    if (gid >= total) return;
-    const uint32_t write_index = (uint32_t)(gid / chunks_per_write);
-    const uint32_t in_write = (uint32_t)(gid - (uint64_t)write_index * chunks_per_write);
+    const uint32_t in_write = blockIdx.y * blockDim.x + threadIdx.x;
+    if (in_write >= p.num_kv_heads * chunks_per_row) return;
     const uint32_t head = in_write / chunks_per_row;
     const uint32_t dim = (in_write - head * chunks_per_row) * 8;
 
@@ -69,14 +69,8 @@ __global__ __launch_bounds__(256) void kv_page_write_kernel(const PageWriteParam
         const uint4 v = *reinterpret_cast<const uint4*>(p.flat_v + source);
         if constexpr (FP8_PAGES) {
             auto encode8 = [](uint4 bits) {
-                const uint32_t words[4] = {bits.x, bits.y, bits.z, bits.w};
-                uint32_t codes[2] = {0u, 0u};
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const uint32_t value = (words[i >> 1] >> ((i & 1) * 16)) & 0xffffu;
-                    codes[i >> 2] |= bf16_bits_to_fp8_e4m3fn(value) << ((i & 3) * 8);
-                }
-                return make_uint2(codes[0], codes[1]);
+                return make_uint2(bf16x2_bits_to_fp8x2_e4m3fn(bits.x) | (bf16x2_bits_to_fp8x2_e4m3fn(bits.y) << 16),
+                                  bf16x2_bits_to_fp8x2_e4m3fn(bits.z) | (bf16x2_bits_to_fp8x2_e4m3fn(bits.w) << 16));
             };
             *reinterpret_cast<uint2*>(k_target) = encode8(k);
             *reinterpret_cast<uint2*>(v_target) = encode8(v);
@@ -110,9 +104,18 @@ __global__ __launch_bounds__(256) void fp8_decode_kernel(const uint8_t* codes, u
     for (uint64_t i = gid; i < count; ++i) bf16_out[i] = (uint16_t)(fp8x2_to_bf16x2<false>(codes[i]) & 0xffffu);
 }
 
+// Thread t encodes elements 2t and 2t+1 with the paired hardware conversion the page writer uses; a last odd element
+// takes the integer encoder.
 __global__ __launch_bounds__(256) void fp8_encode_kernel(const uint16_t* bf16_in, uint8_t* codes, uint64_t count) {
-    const uint64_t gid = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-    if (gid < count) codes[gid] = (uint8_t)bf16_bits_to_fp8_e4m3fn(bf16_in[gid]);
+    const uint64_t gid = ((uint64_t)blockIdx.x * 256 + threadIdx.x) * 2;
+    if (gid + 1 < count) {
+        const uint32_t pair = (uint32_t)bf16_in[gid] | ((uint32_t)bf16_in[gid + 1] << 16);
+        const uint32_t both = bf16x2_bits_to_fp8x2_e4m3fn(pair);
+        codes[gid] = (uint8_t)(both & 0xffu);
+        codes[gid + 1] = (uint8_t)(both >> 8);
+    } else if (gid < count) {
+        codes[gid] = (uint8_t)bf16_bits_to_fp8_e4m3fn(bf16_in[gid]);
+    }
 }
 
 static DeviceReplayU32 to_device_replay(khm_replay_u32 value) { return DeviceReplayU32{value.is_parameter, value.value}; }
@@ -202,12 +205,15 @@ extern "C" int khm_kv_page_write(const khm_kv_page_write_config* config, const k
     p.num_gqa_layers = layout.num_gqa_layers;
     p.num_blocks = layout.num_blocks;
     p.num_page_ids_per_block = layout.num_page_ids_per_block;
-    const uint64_t chunks = (uint64_t)shape->num_total_token_writes * config->num_kv_heads * ((config->head_dim + 7) / 8);
-    const uint32_t blocks = (uint32_t)((chunks + 255) / 256);
+    const uint64_t chunks_per_write = (uint64_t)config->num_kv_heads * ((config->head_dim + 7) / 8);
+    const uint32_t block_threads = (uint32_t)(chunks_per_write >= 1024 ? 1024 : (chunks_per_write + 63) / 64 * 64);
+    const uint64_t chunk_blocks = (chunks_per_write + block_threads - 1) / block_threads;
+    KHM_REQUIRE(chunk_blocks <= 65535, "GQA KV page write: %llu chunks per token write exceed the launch grid", (unsigned long long)chunks_per_write);
+    const dim3 grid(shape->num_total_token_writes, (uint32_t)chunk_blocks);
     if (config->kv_dtype == KHM_DTYPE_FP8_E4M3FN) {
-        hipLaunchKernelGGL(kv_page_write_kernel<true>, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+        hipLaunchKernelGGL(kv_page_write_kernel<true>, grid, dim3(block_threads), 0, static_cast<hipStream_t>(stream), p);
     } else {
-        hipLaunchKernelGGL(kv_page_write_kernel<false>, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+        hipLaunchKernelGGL(kv_page_write_kernel<false>, grid, dim3(block_threads), 0, static_cast<hipStream_t>(stream), p);
     }
     return check_page_write_launch("KV page write");
 }
@@ -234,7 +240,7 @@ extern "C" int khm_bf16_to_fp8_e4m3_device(khm_buffer bf16_in, khm_buffer codes,
                 (unsigned long long)bf16_in.len_bytes, (unsigned long long)(count * 2));
     KHM_REQUIRE(codes.ptr != nullptr && codes.len_bytes >= count, "codes buffer holds %llu bytes, needs %llu",
                 (unsigned long long)codes.len_bytes, (unsigned long long)count);
-    hipLaunchKernelGGL(fp8_encode_kernel, dim3((uint32_t)((count + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+    hipLaunchKernelGGL(fp8_encode_kernel, dim3((uint32_t)(((count + 1) / 2 + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint16_t*>(bf16_in.ptr), static_cast<uint8_t*>(codes.ptr), count);
     return check_page_write_launch("FP8 encode");
 }
