@@ -31,7 +31,7 @@ NUM_POOLS = 3
 # HBM bytes per Map launch from the hardware counters, (FETCH_SIZE * 2.000 + WRITE_SIZE * 1.000) KiB per dispatch:
 # two `rocprofv3 --pmc` runs per config, each counter scaled by what it reads for a plain 1 GiB copy kernel
 # (`--calibration-copy`).  The summaries with their commands are the text files under profiles/.
-MEASURED_MAP_TRAFFIC_BYTES = {2: 567_672_053, 3: 2_152_169_472, 4: 1_450_895_667, 5: 2_561_668_096}
+MEASURED_MAP_TRAFFIC_BYTES = {2: 564_411_624, 3: 2_151_730_601, 4: 1_450_884_731, 5: 2_541_369_749}
 
 CONFIGS = {
     1: dict(name="config1: B=1 q=1 Hq32/Hkv8/D128 ctx 1024, identity pages", hq=32, hkv=8, d=128, kind="decode", kv_slice=64),
@@ -470,6 +470,8 @@ def main() -> int:
     parser.add_argument("--config", type=int, default=2, help="headline config (default 2)")
     parser.add_argument("--only", action="store_true", help="time only the headline config (used for profiling runs)")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    parser.add_argument("--producers", action="store_true",
+                        help="time only the kernels that feed the SDPA (RMSNorm + RoPE, K/V page write) and print their JSON (profiling runs)")
     parser.add_argument("--calibration-copy", action="store_true",
                         help="also launch a plain 1 GiB copy kernel, the known-size reference for FETCH_SIZE / WRITE_SIZE counter runs")
     args = parser.parse_args()
@@ -485,6 +487,9 @@ def main() -> int:
     device = torch.device("cuda:0")
     if args.calibration_copy:
         calibration_copy(device)
+    if args.producers:
+        print(json.dumps({"producers": producer_rows(device, steps=max(args.steps, 1))}))
+        return 0
     headline = Workload(args.config, device)
     head = headline.report(args.steps, args.warmup)
     others = {}
