@@ -596,6 +596,40 @@ int khm_gqa_metadata_compute(const uint32_t* req_slots, const uint32_t* token_in
                              uint32_t* q_token_ranges, uint32_t* sdpa_map_task_templates,
                              uint32_t* cu_sdpa_partial_outputs, uint64_t token_capacity, uint64_t template_capacity);
 
+/* ------------------------------------------------------------------------------------------
+ * Block (DFlash2 proposal) attention, host side: every Q-token range reduces its history split-KV partials plus one dense
+ * block partial (khm_bidi_block_sdpa writes it into the last slot of the range).  Pure host logic, no device calls.
+ * ------------------------------------------------------------------------------------------ */
+/* BiDiBlockCapacity (inference-executor-core/src/attn/gqa/bidi_block_gqa_core.rs:27-63) + BiDiBlockGQACapacity
+ * (inference-executor-metal/src/attn/bidi_block_gqa/capacity.rs:7-48). */
+typedef struct khm_bidi_block_capacity {
+    uint32_t max_requests;
+    uint32_t block_size;
+    uint32_t max_tokens;
+    uint32_t max_q_tokens;
+    uint32_t max_q_token_ranges;
+    uint32_t max_sdpa_map_task_templates;
+    uint64_t max_sdpa_partial_state_groups;
+} khm_bidi_block_capacity;
+int khm_bidi_block_capacity_new(uint32_t max_requests, uint32_t block_size, uint32_t max_q_tokens, khm_bidi_block_capacity* out);
+/* bidi_block_gqa::sdpa::Selector::select (attn/bidi_block_gqa/sdpa.rs:46-110): the registry variant that loads the
+ * history K/V least often for a fixed block width, and the capacity that goes with it. */
+int khm_bidi_block_select(const khm_sdpa_config* config, uint32_t max_requests, uint32_t block_size, khm_sdpa_variant* variant,
+                          khm_bidi_block_capacity* capacity);
+/* BiDiBlockGQAMetadata::new (bidi_block_gqa_core.rs:77-139) + build_metal_metadata and
+ * BiDiBlockGQAMetadataBuffers::update_with_active_requests (attn/bidi_block_gqa/metadata.rs:87-147,182-375).
+ * Inputs: req_slots [R] (unique), and per block row (R * block_size rows) the query token index and its nonempty visible
+ * history range.  Outputs (host arrays): req_slots_by_token / flat_token_indices [T], visible_kv_token_ranges [T][2],
+ * q_token_ranges [ranges][2], sdpa_map_task_templates [max_sdpa_map_task_templates][3] (written up to the replay
+ * capacity, padded with u32::MAX; each range's last template is the u32::MAX placeholder of its block partial),
+ * cu_sdpa_partial_outputs [ranges + 1], and the replay shape of the first num_active_requests requests. */
+int khm_bidi_block_metadata_compute(const uint32_t* req_slots, uint32_t num_requests, const uint32_t* flat_query_token_indices,
+                                    const uint32_t* history_token_begins, const uint32_t* history_token_ends, uint32_t block_size,
+                                    const khm_sdpa_variant* variant, uint32_t max_sdpa_map_task_templates,
+                                    uint32_t num_active_requests, uint32_t* req_slots_by_token, uint32_t* flat_token_indices,
+                                    uint32_t* visible_kv_token_ranges, uint32_t* q_token_ranges, uint32_t* sdpa_map_task_templates,
+                                    uint32_t* cu_sdpa_partial_outputs, khm_gqa_replay_shape* out_shape);
+
 #ifdef __cplusplus
 }
 #endif

@@ -199,6 +199,13 @@ class BidiBlockSdpaBuffers(ctypes.Structure):
                 ("partial_exp_sums", Buffer), ("partial_max_logits", Buffer), ("partial_output", Buffer)]
 
 
+class BidiBlockCapacity(ctypes.Structure):
+    """`BiDiBlockCapacity` + `BiDiBlockGQACapacity`."""
+
+    _fields_ = [("max_requests", u32), ("block_size", u32), ("max_tokens", u32), ("max_q_tokens", u32), ("max_q_token_ranges", u32),
+                ("max_sdpa_map_task_templates", u32), ("max_sdpa_partial_state_groups", u64)]
+
+
 class RopeScalingStruct(ctypes.Structure):
     """`rms_norm_rope::RopeScaling`; kind 0 = default, 1 = Yarn."""
 
@@ -234,6 +241,7 @@ EXPORTED_SYMBOLS = (
     "khm_fp8_e4m3_to_bf16_device", "khm_bf16_to_fp8_e4m3_device",
     "khm_kv_page_write_num_tokens_per_page", "khm_kv_page_write",
     "khm_bidi_block_sdpa",
+    "khm_bidi_block_capacity_new", "khm_bidi_block_select", "khm_bidi_block_metadata_compute",
     "khm_rms_norm_rope_yarn_correction_range", "khm_rms_norm_rope_kernel_parameters", "khm_rms_norm_rope",
     "khm_replay_bucket_policy_create", "khm_replay_bucket_policy_destroy", "khm_replay_bucket_policy_max_capacity",
     "khm_replay_bucket_policy_buckets", "khm_replay_bucket_policy_capacity", "khm_replay_bucket_policy_capacity_allow_zero",
@@ -316,6 +324,11 @@ def lib() -> ctypes.CDLL:
                                          ctypes.POINTER(KvPageWriteBuffers), ReplayU32, ReplayU32, ctypes.c_void_p, ctypes.c_void_p]
     handle.khm_bidi_block_sdpa.argtypes = [ctypes.POINTER(BidiBlockSdpaConfig), ctypes.POINTER(BidiBlockSdpaShape),
                                            ctypes.POINTER(BidiBlockSdpaBuffers), ReplayU32, ctypes.c_void_p, ctypes.c_void_p]
+    u32_p = ctypes.POINTER(u32)
+    handle.khm_bidi_block_capacity_new.argtypes = [u32, u32, u32, ctypes.POINTER(BidiBlockCapacity)]
+    handle.khm_bidi_block_select.argtypes = [ctypes.POINTER(SdpaConfig), u32, u32, ctypes.POINTER(SdpaVariant), ctypes.POINTER(BidiBlockCapacity)]
+    handle.khm_bidi_block_metadata_compute.argtypes = [u32_p, u32, u32_p, u32_p, u32_p, u32, ctypes.POINTER(SdpaVariant), u32, u32, u32_p, u32_p,
+                                                       u32_p, u32_p, u32_p, u32_p, ctypes.POINTER(GqaReplayShape)]
     float_p = ctypes.POINTER(ctypes.c_float)
     handle.khm_rms_norm_rope_yarn_correction_range.argtypes = [ctypes.POINTER(RmsNormRopeConfig), float_p, float_p]
     handle.khm_rms_norm_rope_kernel_parameters.argtypes = [ctypes.POINTER(RmsNormRopeConfig), float_p, u32, float_p]

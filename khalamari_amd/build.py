@@ -21,6 +21,7 @@ SOURCES = [
     "replay_bucket_policy.cpp",
     "selector.cpp",
     "batch_metadata.cpp",
+    "bidi_block_metadata.cpp",
     "components.hip",
     "kv_page_write.hip",
     "bidi_block_sdpa.hip",

@@ -195,3 +195,95 @@ def test_gpu_history_and_block_composite(device, visible_begins):
         weights = np.exp(scores - scores.max())
         expected = weights @ values / weights.sum()
         assert np.abs(actual[token] - expected[None, :]).max() < 1e-2, (token, actual[token, 0, :4], expected[:4])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fp8_pages,window", [(False, 0xFFFFFFFF), (True, 64)])
+def test_gpu_spec_decode_step_from_selected_variant_and_built_metadata(device, fp8_pages, window):
+    """A whole proposal step the way the executor drives it (attn/bidi_block_gqa/backend.rs:394-480): variant and capacity
+    from the block selector, metadata from the block metadata builder, history partials from the sliced-Q Map over the
+    paged cache, the dense block partial, and the Reduce; against a float64 softmax over each row's visible history
+    window plus its whole block."""
+    import torch
+
+    from khalamari_amd import bidi_block_metadata as bbm
+    from khalamari_amd import bidi_block_sdpa as bb
+    from khalamari_amd import sdpa, sliced_kv, sliced_q
+    from khalamari_amd._lib import DTYPE_FP8_E4M3FN
+
+    rng = np.random.default_rng(11 + int(fp8_pages))
+    hq, hkv, d, tpp, block_size = 8, 2, 128, 16, 7
+    scale = float(np.float32(d) ** np.float32(-0.5))
+    anchors, slots = [37, 150, 600], [2, 0, 1]                 # history lengths; request slots in batch order
+    sconfig = sdpa.Config(DTYPE_BF16, hq, hkv, d, tpp)
+    variant, capacity = bbm.select(sconfig, len(anchors), block_size)
+    assert variant.map_max_q_tokens == 8 and sdpa.has_kernel(sconfig, variant, DTYPE_FP8_E4M3FN if fp8_pages else DTYPE_BF16)
+    indices, ranges = [], []
+    for anchor in anchors:
+        for offset in range(block_size):
+            indices.append(anchor + offset)
+            ranges.append((max(anchor + offset + 1 - window, 0), anchor))
+    meta = bbm.build(slots, indices, ranges, block_size, variant, capacity.max_sdpa_map_task_templates)
+    shape = meta.replay_shape
+    n = len(indices)
+
+    kv_dtype = oracle.KV_FP8_E4M3FN if fp8_pages else oracle.KV_BF16
+    rounding = oracle.fp8_round_trip if fp8_pages else oracle.bf16_round
+    num_blocks = -(-max(anchors) // tpp)
+    geom = oracle.Geometry(hq, hkv, d, tpp, scale, 1, num_blocks, 1, kv_dtype)
+    histories = [(rounding(rng.standard_normal((a, hkv, d)).astype(np.float32)), rounding(rng.standard_normal((a, hkv, d)).astype(np.float32)))
+                 for a in anchors]
+    pages_per_request = [-(-a // tpp) for a in anchors]
+    order = rng.permutation(sum(pages_per_request) + 3)
+    page_lists, cursor = [], 0
+    for count in pages_per_request:
+        page_lists.append([int(x) for x in order[cursor:cursor + count]])
+        cursor += count
+    pages = oracle.pack_pages(geom, len(order), histories, page_lists, fill_bits=0x7F if fp8_pages else 0x7FC0)   # NaN everywhere else
+    table = np.full((3, num_blocks), 0xFFFFFFFF, dtype=np.uint32)       # indexed by request SLOT
+    for slot, page_list in zip(slots, page_lists):
+        table[slot, :len(page_list)] = page_list
+    q = oracle.bf16_round(rng.standard_normal((n, hq, d)).astype(np.float32))
+    local_k = oracle.bf16_round(rng.standard_normal((n, hkv, d)).astype(np.float32))
+    local_v = oracle.bf16_round(rng.standard_normal((n, hkv, d)).astype(np.float32))
+
+    qconfig = sliced_q.Config(hq, hkv, d, scale, geom.page_bytes, sliced_kv.Layout(3, 1, num_blocks, 1), DTYPE_BF16,
+                              DTYPE_FP8_E4M3FN if fp8_pages else DTYPE_BF16)
+    qshape = sliced_q.Shape(shape.num_total_tokens, shape.num_total_q_token_tiles, shape.num_total_sdpa_map_task_templates)
+    map_compute = sliced_q.Compute.new(qconfig, variant, qshape)
+    dev = lambda a: _to(device, a)  # noqa: E731
+    q_d, ranges_d, cu_d = dev(oracle.f32_to_bf16_bits(q)), dev(meta.q_token_ranges), dev(meta.cu_sdpa_partial_outputs)
+    groups = int(shape.num_total_sdpa_map_task_templates) * int(variant.map_max_q_tokens) * hq
+    sums = torch.full((groups,), float("nan"), dtype=torch.float32, device=device)
+    maxs = torch.full((groups,), float("nan"), dtype=torch.float32, device=device)
+    partial = torch.full((groups * d * 2,), 0xFF, dtype=torch.uint8, device=device)
+    out = torch.zeros(n * hq * d, dtype=torch.int16, device=device)
+    fixed = ReplayU32.fixed
+    map_compute.invoke_map(q=q_d, kv_pages=dev(pages), req_slots=dev(meta.req_slots), page_ids=dev(table),
+                           visible_kv_token_ranges=dev(meta.visible_kv_token_ranges), q_token_ranges=ranges_d,
+                           sdpa_map_task_templates=dev(meta.sdpa_map_task_templates), partial_output=partial, partial_exp_sums=sums,
+                           partial_max_logits=maxs, page_table_index=fixed(0), num_active_tokens=fixed(shape.num_tokens),
+                           num_active_q_token_tiles=fixed(shape.num_q_token_tiles), num_active_kv_splits=fixed(shape.num_sdpa_map_task_templates))
+    bb.Compute(bb.Config(block_size, int(variant.map_max_q_tokens), hq, hkv, d, scale, DTYPE_BF16)).invoke(
+        bb.Shape(shape.num_total_tokens, shape.num_total_q_token_tiles, shape.num_total_sdpa_map_task_templates), fixed(shape.num_q_token_tiles),
+        q=q_d, local_k=dev(oracle.f32_to_bf16_bits(local_k)), local_v=dev(oracle.f32_to_bf16_bits(local_v)), q_token_ranges=ranges_d,
+        cu_sdpa_partial_outputs=cu_d, partial_exp_sums=sums, partial_max_logits=maxs, partial_output=partial)
+    map_compute.invoke_reduce(partial_output=partial, partial_exp_sums=sums, partial_max_logits=maxs, q_token_ranges=ranges_d,
+                              cu_sdpa_partial_outputs=cu_d, output=out, num_active_q_token_tiles=fixed(shape.num_q_token_tiles))
+    torch.cuda.synchronize()
+    actual = oracle.bf16_bits_to_f32(out.cpu().numpy().view(np.uint16)).reshape(n, hq, d)
+    assert np.isfinite(actual).all()
+    for request, anchor in enumerate(anchors):
+        rows = slice(request * block_size, (request + 1) * block_size)
+        for offset in range(block_size):
+            token = request * block_size + offset
+            begin = ranges[token][0]
+            for head in range(hq):
+                kv_head = head // (hq // hkv)
+                keys = np.concatenate([histories[request][0][begin:anchor, kv_head], local_k[rows, kv_head]]).astype(np.float64)
+                values = np.concatenate([histories[request][1][begin:anchor, kv_head], local_v[rows, kv_head]]).astype(np.float64)
+                scores = keys @ q[token, head].astype(np.float64) * scale
+                weights = np.exp(scores - scores.max())
+                expected = weights @ values / weights.sum()
+                error = np.abs(actual[token, head] - expected)
+                assert np.all(error <= 2e-3 + 1e-2 * np.abs(expected)), (request, offset, head, error.max())
