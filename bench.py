@@ -3,7 +3,7 @@
 
 `python bench.py [--gpus 1] [--steps K] [--warmup W]` prints ONE JSON line.  A step is one pass of the
 hot path (Map + Reduce, or the direct Map) over one batch of synthetic input that already sits in HBM.
-The headline workload is BASELINE config 2 (32 ragged decode requests, 512-token split-KV partitions);
+The headline workload is config 2 (32 ragged decode requests, 512-token split-KV partitions);
 the other synthetic configs are timed briefly and reported under "configs".
 
 Inputs: Q/K/V ~ N(0,1) rounded to bf16 (generated on the device, fixed seeds), context lengths and page
@@ -93,7 +93,7 @@ class Workload:
         for r, n in enumerate(pages_per_request):
             table[r, :n] = order[cursor:cursor + n]
             cursor += n
-        # FP8 E4M3FN pages (the reference's cache format, 32 KiB at these geometries) or bf16 pages (the BASELINE configs)
+        # FP8 E4M3FN pages (the reference's cache format, 32 KiB at these geometries) or bf16 pages (what the five benchmark configs are defined on)
         self.fp8_pages = fp8_pages
         self.kv_element_bytes = 1 if fp8_pages else 2
         kv_dtype = DTYPE_FP8_E4M3FN if fp8_pages else DTYPE_BF16

@@ -21,7 +21,7 @@ def _decode_case(device, *, hq, hkv, d, tpp, histories, kv_slice, seed, partial_
 
 
 def test_config1_single_sequence_identity_pages(device):
-    """BASELINE config 1: batch 1, Hq32/Hkv8/D128, context 1024, page 16, identity page table."""
+    """Benchmark config 1: batch 1, Hq32/Hkv8/D128, context 1024, page 16, identity page table."""
     stats = _decode_case(device, hq=32, hkv=8, d=128, tpp=16, histories=[1023], kv_slice=256, seed=1, permute=False)
     print(stats)
 

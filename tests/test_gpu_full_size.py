@@ -1,4 +1,4 @@
-"""Parity at the full BASELINE sizes.  The synthetic configs are built exactly as bench.py builds them (same seeds,
+"""Parity at the full sizes of the five benchmark configs.  The synthetic configs are built exactly as bench.py builds them (same seeds,
 page permutations and selector decisions), one step runs through the C ABI, and the output rows of sampled Q tokens are
 checked against the CPU oracle at the full context - every token where that takes seconds (configs 2 and 3), the
 first / middle / last token of each request otherwise (as the reference's bench gate samples them:
