@@ -148,8 +148,11 @@ __device__ __forceinline__ float value_of_lane_xor(float v, uint32_t lane) {
 // kRowsInFlight rows it visits, whose loads are all issued before the first is used.
 constexpr int kRowsInFlight = 8;
 
-template <typename T, typename W>
-__global__ __launch_bounds__(256) void rms_norm_rope_rows_kernel(const RmsNormRopeParams p, const uint32_t lanes_per_row) {
+// LPR (lanes per row) and PARTNER (lanes between an element and its rotary partner: 16 or 32 for the VALU swaps, 0 for
+// any other distance through a generic shuffle) are compile-time, so the row loop is straight-line code.
+template <typename T, typename W, uint32_t LPR, uint32_t PARTNER>
+__global__ __launch_bounds__(256) void rms_norm_rope_rows_kernel(const RmsNormRopeParams p) {
+    constexpr uint32_t lanes_per_row = LPR;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
     const uint32_t token = blockIdx.x;
@@ -189,7 +192,7 @@ __global__ __launch_bounds__(256) void rms_norm_rope_rows_kernel(const RmsNormRo
         Row4<float>::unpack(*reinterpret_cast<const float4*>(sines + pair), sine);
         Row4<float>::unpack(*reinterpret_cast<const float4*>(cosines + pair), cosine);
     }
-    const uint32_t partner_distance = rope_half / 4;
+    const float inverse_dim = 1.0f / (float)p.head_dim;
 #pragma unroll
     for (int j = 0; j < kRowsInFlight; ++j) {
         float x[4];
@@ -198,9 +201,12 @@ __global__ __launch_bounds__(256) void rms_norm_rope_rows_kernel(const RmsNormRo
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc += x[i] * x[i];
         acc = sum_in_row16(acc);
-        if (lanes_per_row >= 32) acc += value_of_lane_xor<16>(acc, lane);
-        if (lanes_per_row == 64) acc += value_of_lane_xor<32>(acc, lane);
-        const float inv_rms = 1.0f / sqrtf(acc / (float)p.head_dim + p.eps);
+        if constexpr (LPR >= 32) acc += value_of_lane_xor<16>(acc, lane);
+        if constexpr (LPR == 64) acc += value_of_lane_xor<32>(acc, lane);
+        // v_rsq_f32 (1 ulp) and one Newton step, which leaves the error below that of a correctly rounded rsqrt's input
+        const float mean = acc * inverse_dim + p.eps;
+        float inv_rms = __builtin_amdgcn_rsqf(mean);
+        inv_rms = inv_rms * __builtin_fmaf(-0.5f * mean * inv_rms, inv_rms, 1.5f);
         float out[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -210,8 +216,10 @@ __global__ __launch_bounds__(256) void rms_norm_rope_rows_kernel(const RmsNormRo
             } else {
                 normed = w[i] * x[i] * inv_rms;
             }
-            const float partner = partner_distance == 16 ? value_of_lane_xor<16>(normed, lane)
-                                  : partner_distance == 32 ? value_of_lane_xor<32>(normed, lane) : __shfl(normed, partner_lane);
+            float partner;
+            if constexpr (PARTNER == 16) partner = value_of_lane_xor<16>(normed, lane);
+            else if constexpr (PARTNER == 32) partner = value_of_lane_xor<32>(normed, lane);
+            else partner = __shfl(normed, partner_lane);
             out[i] = normed;
             if (rotated) {
                 out[i] = lower ? p.attention_factor * (normed * cosine[i] - partner * sine[i])
@@ -366,10 +374,23 @@ extern "C" int khm_rms_norm_rope(const khm_rms_norm_rope_config* config, uint32_
         const uint32_t lanes_per_row = config->head_dim <= 64 ? 16u : (config->head_dim <= 128 ? 32u : 64u);
         const uint32_t heads_per_block = 4 * kRowsInFlight * (64u / lanes_per_row);
         const dim3 grid(num_total_tokens, (config->num_heads + heads_per_block - 1) / heads_per_block);
-        if (io_bf16 && weight_bf16) hipLaunchKernelGGL((rms_norm_rope_rows_kernel<uint16_t, uint16_t>), grid, dim3(256), 0, hip_stream, p, lanes_per_row);
-        else if (io_bf16) hipLaunchKernelGGL((rms_norm_rope_rows_kernel<uint16_t, float>), grid, dim3(256), 0, hip_stream, p, lanes_per_row);
-        else if (weight_bf16) hipLaunchKernelGGL((rms_norm_rope_rows_kernel<float, uint16_t>), grid, dim3(256), 0, hip_stream, p, lanes_per_row);
-        else hipLaunchKernelGGL((rms_norm_rope_rows_kernel<float, float>), grid, dim3(256), 0, hip_stream, p, lanes_per_row);
+        const uint32_t partner_distance = config->rope_dim / 8;   // lanes between the halves of a rotary pair
+        const uint32_t partner = partner_distance == 16 || partner_distance == 32 ? partner_distance : 0;
+        auto launch = [&](auto io_tag, auto weight_tag) {
+            typedef decltype(io_tag) T;
+            typedef decltype(weight_tag) W;
+#define KHM_ROWS_CASE(LPR, PARTNER)                                                                                        \
+    if (lanes_per_row == LPR && partner == PARTNER) {                                                                      \
+        hipLaunchKernelGGL((rms_norm_rope_rows_kernel<T, W, LPR, PARTNER>), grid, dim3(256), 0, hip_stream, p);             \
+        return;                                                                                                            \
+    }
+            KHM_ROWS_CASE(16, 0) KHM_ROWS_CASE(32, 0) KHM_ROWS_CASE(32, 16) KHM_ROWS_CASE(64, 0) KHM_ROWS_CASE(64, 16) KHM_ROWS_CASE(64, 32)
+#undef KHM_ROWS_CASE
+        };
+        if (io_bf16 && weight_bf16) launch(uint16_t{}, uint16_t{});
+        else if (io_bf16) launch(uint16_t{}, float{});
+        else if (weight_bf16) launch(float{}, uint16_t{});
+        else launch(float{}, float{});
     } else {
         const dim3 grid((uint32_t)rows);
         if (io_bf16 && weight_bf16) hipLaunchKernelGGL((rms_norm_rope_kernel<uint16_t, uint16_t>), grid, dim3(64), 0, hip_stream, p);
