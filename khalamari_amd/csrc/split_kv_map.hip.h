@@ -53,10 +53,12 @@ struct MapSmem {
     static constexpr int kVBytes = NWAVES * 16 * kVRowBytes;
     static constexpr int kCols = NT * 16;
     static constexpr int kORowFloats = D + 4;
-    static constexpr int kOBytes = kCols * kORowFloats * 4;
+    // one merged tile, or (one column tile) a tile per wave so that all waves hand over their accumulators at once
+    static constexpr bool kTilePerWave = (NT == 1);
+    static constexpr int kOBytes = (kTilePerWave ? NWAVES : 1) * kCols * kORowFloats * 4;
     static constexpr int kUnionBytes = kVBytes > kOBytes ? kVBytes : kOBytes;
     static constexpr int kQRowBytes = D * 2 + 16;
-    static constexpr int kQBytes = kCols * kQRowBytes;
+    static constexpr int kQBytes = NT == 1 ? 0 : kCols * kQRowBytes;   // a single column tile keeps Q in registers
     static constexpr int kStatsBytes = (NWAVES + 1) * kCols * 3 * 4;   // (reference, sum, maximum) per wave and column
     static constexpr int kTotal = kUnionBytes + kQBytes + kStatsBytes;
 };
@@ -501,20 +503,28 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
             stats_lds[(NWAVES * COLS + c) * 3 + 1] = global_sum > 0.0f ? global_sum * fast_exp2(global_ref - global_max) : 0.0f;
         }
     }
-    for (int w = 0; w < NWAVES; ++w) {
-        if (wave == w) {
+    if constexpr (Smem::kTilePerWave) {
+        // every wave stores its scaled accumulator into a tile of its own; the writer below adds the tiles up
+        float* tile = o_lds + wave * (COLS * Smem::kORowFloats);
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
+        for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<f32x4*>(tile + r16 * Smem::kORowFloats + mt * 16 + g * 4) = acc[0][mt];
+        __syncthreads();
+    } else {
+        for (int w = 0; w < NWAVES; ++w) {
+            if (wave == w) {
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) {
-                    float* cell = o_lds + (nt * 16 + r16) * Smem::kORowFloats + mt * 16 + g * 4;
-                    f32x4 value = acc[nt][mt];
-                    if (w > 0) value += *reinterpret_cast<const f32x4*>(cell);
-                    *reinterpret_cast<f32x4*>(cell) = value;
+                for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) {
+                        float* cell = o_lds + (nt * 16 + r16) * Smem::kORowFloats + mt * 16 + g * 4;
+                        f32x4 value = acc[nt][mt];
+                        if (w > 0) value += *reinterpret_cast<const f32x4*>(cell);
+                        *reinterpret_cast<f32x4*>(cell) = value;
+                    }
                 }
             }
+            __syncthreads();
         }
-        __syncthreads();
     }
 
     // ---- write the block's partial state or final output ------------------------------------
@@ -526,7 +536,11 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
         const uint32_t token_offset = c / p.max_q_heads;
         const uint32_t local_head = c - token_offset * p.max_q_heads;
         if (token_offset >= num_q || local_head >= num_heads) continue;
-        const f32x4 value = *reinterpret_cast<const f32x4*>(o_lds + c * Smem::kORowFloats + d);
+        f32x4 value = *reinterpret_cast<const f32x4*>(o_lds + c * Smem::kORowFloats + d);
+        if constexpr (Smem::kTilePerWave) {
+#pragma unroll
+            for (int w = 1; w < NWAVES; ++w) value += *reinterpret_cast<const f32x4*>(o_lds + (w * COLS + c) * Smem::kORowFloats + d);
+        }
         const uint32_t q_head = first_q_head + local_head;
         uint64_t state;
         if (mode == kMapDirectBf16) {
