@@ -94,24 +94,30 @@ __global__ __launch_bounds__(64) void rms_norm_rope_kernel(const RmsNormRopePara
     }
 }
 
+// Eight consecutive elements of a row as one lane holds them.
 template <typename T>
-struct Row4;
+struct Row8;
 template <>
-struct Row4<float> {
-    using Vec = float4;
-    static __device__ __forceinline__ void unpack(const Vec& v, float (&x)[4]) { x[0] = v.x, x[1] = v.y, x[2] = v.z, x[3] = v.w; }
-    static __device__ __forceinline__ Vec pack(const float (&x)[4]) { return make_float4(x[0], x[1], x[2], x[3]); }
+struct Row8<float> {
+    static __device__ __forceinline__ void load(const float* source, float (&x)[8]) {
+        const float4 a = *reinterpret_cast<const float4*>(source), b = *reinterpret_cast<const float4*>(source + 4);
+        x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w, x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
+    }
+    static __device__ __forceinline__ void store(float* target, const float (&x)[8]) {
+        *reinterpret_cast<float4*>(target) = make_float4(x[0], x[1], x[2], x[3]);
+        *reinterpret_cast<float4*>(target + 4) = make_float4(x[4], x[5], x[6], x[7]);
+    }
 };
 template <>
-struct Row4<uint16_t> {
-    using Vec = uint2;
-    static __device__ __forceinline__ void unpack(const Vec& v, float (&x)[4]) {
-        x[0] = bf16_bits_to_f32((uint16_t)(v.x & 0xffffu)), x[1] = bf16_bits_to_f32((uint16_t)(v.x >> 16));
-        x[2] = bf16_bits_to_f32((uint16_t)(v.y & 0xffffu)), x[3] = bf16_bits_to_f32((uint16_t)(v.y >> 16));
+struct Row8<uint16_t> {
+    static __device__ __forceinline__ void load(const uint16_t* source, float (&x)[8]) {
+        const uint4 v = *reinterpret_cast<const uint4*>(source);
+        const uint32_t words[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[2 * i] = __uint_as_float(words[i] << 16), x[2 * i + 1] = __uint_as_float(words[i] & 0xffff0000u);
     }
-    static __device__ __forceinline__ Vec pack(const float (&x)[4]) {
-        return make_uint2((uint32_t)f32_to_bf16_bits(x[0]) | ((uint32_t)f32_to_bf16_bits(x[1]) << 16),
-                          (uint32_t)f32_to_bf16_bits(x[2]) | ((uint32_t)f32_to_bf16_bits(x[3]) << 16));
+    static __device__ __forceinline__ void store(uint16_t* target, const float (&x)[8]) {
+        *reinterpret_cast<uint4*>(target) = make_uint4(pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3]), pack_bf16x2(x[4], x[5]), pack_bf16x2(x[6], x[7]));
     }
 };
 
@@ -119,14 +125,6 @@ struct Row4<uint16_t> {
 template <int CTRL>
 __device__ __forceinline__ float dpp_move(float v) {
     return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), CTRL, 0xf, 0xf, true));
-}
-// Sum over the 16 lanes of a row, in every lane: quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror.
-__device__ __forceinline__ float sum_in_row16(float v) {
-    v += dpp_move<0xB1>(v);
-    v += dpp_move<0x4E>(v);
-    v += dpp_move<0x141>(v);
-    v += dpp_move<0x140>(v);
-    return v;
 }
 // The value lane (l ^ 16) holds (ROWS = 16) or lane (l ^ 32) holds (ROWS = 32).
 template <int ROWS>
@@ -140,42 +138,50 @@ __device__ __forceinline__ float value_of_lane_xor(float v, uint32_t lane) {
         return __uint_as_float((lane & 32u) ? halves[0] : halves[1]);
     }
 }
+// Sum over the LPR lanes of a row (8, 16, 32 or 64 aligned lanes), in every lane: quad_perm [1,0,3,2], quad_perm [2,3,0,1],
+// row_half_mirror, then row_mirror and the row swaps as far as the row reaches.
+template <uint32_t LPR>
+__device__ __forceinline__ float sum_in_row(float v, uint32_t lane) {
+    v += dpp_move<0xB1>(v);
+    v += dpp_move<0x4E>(v);
+    v += dpp_move<0x141>(v);
+    if constexpr (LPR >= 16) v += dpp_move<0x140>(v);
+    if constexpr (LPR >= 32) v += value_of_lane_xor<16>(v, lane);
+    if constexpr (LPR == 64) v += value_of_lane_xor<32>(v, lane);
+    return v;
+}
 
-// The same arithmetic for head_dim <= 256 with head_dim and rope_dim / 2 multiples of 4.  A row occupies
-// LPR = 16, 32 or 64 lanes (4 elements per lane from one vector load), so a wavefront holds 64 / LPR rows side by side;
-// the rotary partner (rope_dim / 2 elements away) is the same slot of the lane rope_dim / 8 away.  A block serves up
-// to 16 * 64 / LPR heads of ONE token: each lane evaluates the token's sines and cosines once and reuses them for the
-// kRowsInFlight rows it visits, whose loads are all issued before the first is used.
-constexpr int kRowsInFlight = 8;
+// The same arithmetic for head_dim <= 512 with head_dim and rope_dim / 2 multiples of 8.  A row occupies LPR = 8, 16, 32
+// or 64 lanes (8 elements per lane from one 16- or 32-byte load), so a wavefront holds 64 / LPR rows side by side; the
+// rotary partner (rope_dim / 2 elements away) is the same slot of the lane PARTNER = rope_dim / 16 away: 8 lanes is a
+// DPP row rotation, 16 and 32 the row swaps, anything else (PARTNER = 0) a generic shuffle.  A block serves the heads
+// of ONE token: the first lanes evaluate the token's sines and cosines once into LDS, and each wave issues the loads
+// of up to kRowsInFlight row groups before it uses the first.
+constexpr int kRowsInFlight = 4;
 
-// LPR (lanes per row) and PARTNER (lanes between an element and its rotary partner: 16 or 32 for the VALU swaps, 0 for
-// any other distance through a generic shuffle) are compile-time, so the row loop is straight-line code.
 template <typename T, typename W, uint32_t LPR, uint32_t PARTNER>
 __global__ __launch_bounds__(256) void rms_norm_rope_rows_kernel(const RmsNormRopeParams p) {
-    constexpr uint32_t lanes_per_row = LPR;
+    constexpr uint32_t kRowsPerWave = 64u / LPR;
+    constexpr uint32_t kHeadsPerBlock = 4 * kRowsInFlight * kRowsPerWave;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
     const uint32_t token = blockIdx.x;
     if (token >= resolve_u32(p.num_active_tokens, p.replay_parameters)) return;
-    const uint32_t rows_per_wave = 64u / lanes_per_row;
-    const uint32_t sub_row = lane / lanes_per_row;
-    const uint32_t first = (lane % lanes_per_row) * 4;
+    const uint32_t sub_row = lane / LPR;
+    const uint32_t first = (lane % LPR) * 8;
     const bool holds = first < p.head_dim;
     const uint32_t rope_half = p.rope_dim / 2;
     const bool lower = first < rope_half, rotated = first < p.rope_dim;
-    const int partner_lane = ((int)lane + (lower ? (int)(rope_half / 4) : -(int)(rope_half / 4))) & 63;
+    const int partner_lane = ((int)lane + (lower ? (int)(rope_half / 8) : -(int)(rope_half / 8))) & 63;
 
-    using Vec = typename Row4<T>::Vec;
-    const uint32_t heads_per_block = 4 * kRowsInFlight * rows_per_wave;
-    Vec raw[kRowsInFlight];
+    float x[kRowsInFlight][8];
     uint32_t heads[kRowsInFlight];
 #pragma unroll
     for (int j = 0; j < kRowsInFlight; ++j) {
-        heads[j] = blockIdx.y * heads_per_block + (j * 4 + wave) * rows_per_wave + sub_row;
-        raw[j] = Vec{};
-        if (holds && heads[j] < p.num_heads) {
-            raw[j] = *reinterpret_cast<const Vec*>(static_cast<const T*>(p.input) + ((uint64_t)token * p.num_heads + heads[j]) * p.head_dim + first);
-        }
+        heads[j] = blockIdx.y * kHeadsPerBlock + (j * 4 + wave) * kRowsPerWave + sub_row;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[j][i] = 0.0f;
+        if (holds && heads[j] < p.num_heads) Row8<T>::load(static_cast<const T*>(p.input) + ((uint64_t)token * p.num_heads + heads[j]) * p.head_dim + first, x[j]);
     }
     // the token's rotation table, one sine/cosine evaluation per rotary pair for the whole block
     __shared__ __align__(16) float sines[kMaxRopeHalf];
@@ -184,40 +190,39 @@ __global__ __launch_bounds__(256) void rms_norm_rope_rows_kernel(const RmsNormRo
         const float position = (float)p.flat_token_indices[token];
         sincosf(position * p.inverse_frequencies[threadIdx.x], &sines[threadIdx.x], &cosines[threadIdx.x]);
     }
-    float w[4] = {0.0f, 0.0f, 0.0f, 0.0f}, sine[4] = {0.0f, 0.0f, 0.0f, 0.0f}, cosine[4] = {1.0f, 1.0f, 1.0f, 1.0f};
-    if (holds) Row4<W>::unpack(*reinterpret_cast<const typename Row4<W>::Vec*>(static_cast<const W*>(p.norm_weight) + first), w);
+    float w[8], sine[8], cosine[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w[i] = 0.0f, sine[i] = 0.0f, cosine[i] = 1.0f;
+    if (holds) Row8<W>::load(static_cast<const W*>(p.norm_weight) + first, w);
     __syncthreads();
     if (rotated) {
         const uint32_t pair = lower ? first : first - rope_half;
-        Row4<float>::unpack(*reinterpret_cast<const float4*>(sines + pair), sine);
-        Row4<float>::unpack(*reinterpret_cast<const float4*>(cosines + pair), cosine);
+        Row8<float>::load(sines + pair, sine);
+        Row8<float>::load(cosines + pair, cosine);
     }
     const float inverse_dim = 1.0f / (float)p.head_dim;
 #pragma unroll
     for (int j = 0; j < kRowsInFlight; ++j) {
-        float x[4];
-        Row4<T>::unpack(raw[j], x);
         float acc = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc += x[i] * x[i];
-        acc = sum_in_row16(acc);
-        if constexpr (LPR >= 32) acc += value_of_lane_xor<16>(acc, lane);
-        if constexpr (LPR == 64) acc += value_of_lane_xor<32>(acc, lane);
+        for (int i = 0; i < 8; ++i) acc += x[j][i] * x[j][i];
+        acc = sum_in_row<LPR>(acc, lane);
         // v_rsq_f32 (1 ulp) and one Newton step, which leaves the error below that of a correctly rounded rsqrt's input
         const float mean = acc * inverse_dim + p.eps;
         float inv_rms = __builtin_amdgcn_rsqf(mean);
         inv_rms = inv_rms * __builtin_fmaf(-0.5f * mean * inv_rms, inv_rms, 1.5f);
-        float out[4];
+        float out[8];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 8; ++i) {
             float normed;
             if constexpr (sizeof(T) == 2 && sizeof(W) == 2) {
-                normed = round_to_bf16(w[i] * round_to_bf16(x[i] * inv_rms));
+                normed = round_to_bf16(w[i] * round_to_bf16(x[j][i] * inv_rms));
             } else {
-                normed = w[i] * x[i] * inv_rms;
+                normed = w[i] * x[j][i] * inv_rms;
             }
             float partner;
-            if constexpr (PARTNER == 16) partner = value_of_lane_xor<16>(normed, lane);
+            if constexpr (PARTNER == 8) partner = dpp_move<0x128>(normed);          // row_ror:8 = lane ^ 8 inside a 16-lane row
+            else if constexpr (PARTNER == 16) partner = value_of_lane_xor<16>(normed, lane);
             else if constexpr (PARTNER == 32) partner = value_of_lane_xor<32>(normed, lane);
             else partner = __shfl(normed, partner_lane);
             out[i] = normed;
@@ -226,9 +231,7 @@ __global__ __launch_bounds__(256) void rms_norm_rope_rows_kernel(const RmsNormRo
                                : p.attention_factor * (partner * sine[i] + normed * cosine[i]);
             }
         }
-        if (holds && heads[j] < p.num_heads) {
-            *reinterpret_cast<Vec*>(static_cast<T*>(p.output) + ((uint64_t)token * p.num_heads + heads[j]) * p.head_dim + first) = Row4<T>::pack(out);
-        }
+        if (holds && heads[j] < p.num_heads) Row8<T>::store(static_cast<T*>(p.output) + ((uint64_t)token * p.num_heads + heads[j]) * p.head_dim + first, out);
     }
 }
 
@@ -368,14 +371,15 @@ extern "C" int khm_rms_norm_rope(const khm_rms_norm_rope_config* config, uint32_
     p.eps = config->eps;
     hipStream_t hip_stream = static_cast<hipStream_t>(stream);
     const bool io_bf16 = config->dtype == KHM_DTYPE_BF16, weight_bf16 = config->norm_weight_dtype == KHM_DTYPE_BF16;
-    // vector loads need 16-byte (f32) / 8-byte (bf16) aligned rows; cudaMalloc-style bases and head_dim % 4 == 0 give that
+    // vector loads need 16-byte aligned rows; allocator-aligned bases and head_dim % 8 == 0 give that
     const bool aligned = ((uintptr_t)p.input | (uintptr_t)p.output | (uintptr_t)p.norm_weight) % 16 == 0;
-    if (aligned && config->head_dim <= 256 && config->head_dim % 4 == 0 && (config->rope_dim / 2) % 4 == 0) {
-        const uint32_t lanes_per_row = config->head_dim <= 64 ? 16u : (config->head_dim <= 128 ? 32u : 64u);
+    if (aligned && config->head_dim <= 512 && config->head_dim % 8 == 0 && (config->rope_dim / 2) % 8 == 0) {
+        const uint32_t lanes_per_row = config->head_dim <= 64 ? 8u : (config->head_dim <= 128 ? 16u : (config->head_dim <= 256 ? 32u : 64u));
         const uint32_t heads_per_block = 4 * kRowsInFlight * (64u / lanes_per_row);
         const dim3 grid(num_total_tokens, (config->num_heads + heads_per_block - 1) / heads_per_block);
-        const uint32_t partner_distance = config->rope_dim / 8;   // lanes between the halves of a rotary pair
-        const uint32_t partner = partner_distance == 16 || partner_distance == 32 ? partner_distance : 0;
+        const uint32_t partner_distance = config->rope_dim / 16;   // lanes between the halves of a rotary pair
+        const bool vector_partner = partner_distance == 8 || partner_distance == 16 || partner_distance == 32;
+        const uint32_t partner = vector_partner && partner_distance < lanes_per_row ? partner_distance : 0;
         auto launch = [&](auto io_tag, auto weight_tag) {
             typedef decltype(io_tag) T;
             typedef decltype(weight_tag) W;
@@ -384,7 +388,8 @@ extern "C" int khm_rms_norm_rope(const khm_rms_norm_rope_config* config, uint32_
         hipLaunchKernelGGL((rms_norm_rope_rows_kernel<T, W, LPR, PARTNER>), grid, dim3(256), 0, hip_stream, p);             \
         return;                                                                                                            \
     }
-            KHM_ROWS_CASE(16, 0) KHM_ROWS_CASE(32, 0) KHM_ROWS_CASE(32, 16) KHM_ROWS_CASE(64, 0) KHM_ROWS_CASE(64, 16) KHM_ROWS_CASE(64, 32)
+            KHM_ROWS_CASE(8, 0) KHM_ROWS_CASE(16, 0) KHM_ROWS_CASE(16, 8) KHM_ROWS_CASE(32, 0) KHM_ROWS_CASE(32, 8) KHM_ROWS_CASE(32, 16)
+            KHM_ROWS_CASE(64, 0) KHM_ROWS_CASE(64, 8) KHM_ROWS_CASE(64, 16) KHM_ROWS_CASE(64, 32)
 #undef KHM_ROWS_CASE
         };
         if (io_bf16 && weight_bf16) launch(uint16_t{}, uint16_t{});

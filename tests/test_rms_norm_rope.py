@@ -201,7 +201,8 @@ def test_gpu_reference_known_answers():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("heads,head_dim,rope_dim,yarn", [(32, 128, 128, False), (8, 128, 128, True), (16, 256, 64, False), (3, 80, 40, True), (2, 72, 36, False)])
+@pytest.mark.parametrize("heads,head_dim,rope_dim,yarn", [(32, 128, 128, False), (8, 128, 128, True), (16, 256, 64, False), (3, 80, 40, True), (2, 72, 36, False),
+                                                         (4, 256, 256, False), (4, 256, 128, True), (5, 64, 64, False), (2, 512, 256, False)])
 def test_gpu_f32_rows_match_oracle(heads, head_dim, rope_dim, yarn):
     from khalamari_amd import rms_norm_rope as rnr
 
@@ -223,7 +224,8 @@ def test_gpu_f32_rows_match_oracle(heads, head_dim, rope_dim, yarn):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("heads,head_dim,rope_dim,weight_dtype", [(32, 128, 128, DTYPE_BF16), (8, 128, 128, DTYPE_F32), (16, 256, 64, DTYPE_BF16)])
+@pytest.mark.parametrize("heads,head_dim,rope_dim,weight_dtype", [(32, 128, 128, DTYPE_BF16), (8, 128, 128, DTYPE_F32), (16, 256, 64, DTYPE_BF16),
+                                                                 (6, 256, 256, DTYPE_BF16), (70, 128, 128, DTYPE_BF16)])
 def test_gpu_bf16_rows_match_oracle_and_respect_the_active_count(heads, head_dim, rope_dim, weight_dtype):
     import torch
 
@@ -251,4 +253,7 @@ def test_gpu_bf16_rows_match_oracle_and_respect_the_active_count(heads, head_dim
     magnitude = np.abs(want_f).copy()
     pair = np.hypot(want_f[..., :half], want_f[..., half:rope_dim])
     magnitude[..., :half], magnitude[..., half:rope_dim] = pair, pair
-    assert np.all(np.abs(got_f - want_f) <= np.maximum(magnitude, 2.0 ** -6) * 2.0 ** -7)
+    ulps = np.abs(got_f - want_f) / (np.maximum(magnitude, 2.0 ** -6) * 2.0 ** -7)
+    assert np.mean(ulps <= 1.0) > 0.9999 and ulps.max() <= 2.0, (float(ulps.max()), np.unravel_index(np.argmax(ulps), ulps.shape))
+    # every head, also those of a second block of a token, is as exact as the others
+    assert np.all((got[:active] == want[:active]).mean(axis=(0, 2)) > 0.98)
