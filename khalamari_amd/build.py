@@ -26,6 +26,7 @@ SOURCES = [
     "kv_page_write.hip",
     "bidi_block_sdpa.hip",
     "rms_norm_rope.hip",
+    "calibration.hip",
 ]
 
 HIPCC_FLAGS = [
