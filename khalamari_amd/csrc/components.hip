@@ -13,10 +13,7 @@
 
 namespace khm {
 
-#ifndef KHM_MAP_WAVES
-#define KHM_MAP_WAVES 4
-#endif
-constexpr int kMapWaves = KHM_MAP_WAVES;
+constexpr int kMapWaves = 4;
 
 typedef void (*MapKernel)(const MapParams);
 typedef void (*ReduceKernel)(const ReduceParams);

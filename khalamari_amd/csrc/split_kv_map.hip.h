@@ -63,17 +63,11 @@ struct MapSmem {
     static constexpr int kTotal = kUnionBytes + kQBytes + kStatsBytes;
 };
 
-#ifndef KHM_MAP_PREFETCH
-#define KHM_MAP_PREFETCH 2
-#endif
-#ifdef KHM_MAP_WAVES_PER_EU
-#define KHM_MAP_OCCUPANCY __attribute__((amdgpu_waves_per_eu(KHM_MAP_WAVES_PER_EU, KHM_MAP_WAVES_PER_EU)))
-#else
-#define KHM_MAP_OCCUPANCY
-#endif
+// K/V tiles requested ahead of the one being consumed (register buffers: one more than this).
+constexpr int kMapPrefetchDepth = 2;
 
 template <int D, int NT, int NWAVES, bool KV8 = false>
-__global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_kernel(const MapParams p) {
+__global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapParams p) {
     constexpr int KS = D / 32;
     constexpr int MT = D / 16;
     constexpr int COLS = NT * 16;
@@ -442,7 +436,7 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
     // ---- main loop: a ring of register buffers, loads DEPTH tiles ahead ----------------------
     // Two tiles in flight per wave (8 KB each at D 128 on bf16 pages, half that on FP8 pages, where four in flight were
     // measured slower than two).  The ring is indexed with compile-time constants after unrolling.
-    constexpr int DEPTH = KHM_MAP_PREFETCH;
+    constexpr int DEPTH = kMapPrefetchDepth;
     if (num_wave_tiles > 0) {
         KvTile<D, KV8> ring[DEPTH + 1];
 #pragma unroll
@@ -600,9 +594,6 @@ __global__ __launch_bounds__(NWAVES * 64) KHM_MAP_OCCUPANCY void split_kv_map_ke
     }
     __syncthreads();
     if (flag_lds[0] == 0u) return;
-#ifdef KHM_EXPERIMENT_SKIP_MERGE
-    return;
-#endif
     {
         // Work units are (column, partial-slice) pairs; a group of D/4 lanes owns one unit at a time and walks
         // its partials with an online merge, eight partials' loads in flight at once.  With at least as many

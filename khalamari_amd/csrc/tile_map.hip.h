@@ -28,9 +28,6 @@
 #include "device_params.h"
 #include "fp8_device.hip.h"
 
-#ifndef KHM_X_PRECISE
-#define KHM_X_PRECISE true
-#endif
 namespace khm {
 
 template <int D, int BK, int NSTAGES>
@@ -221,7 +218,7 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     // second MFMA with hi + lo bf16 pairs (the reference keeps P in f32); long contexts, where every weight is small,
     // use one.
     constexpr uint32_t kPreciseSpan = 256;
-    const bool precise = KHM_X_PRECISE && (uint32_t)__builtin_amdgcn_readfirstlane(min_span) <= kPreciseSpan;
+    const bool precise = (uint32_t)__builtin_amdgcn_readfirstlane(min_span) <= kPreciseSpan;
     __syncthreads();   // range_lds is about to be overwritten by the first tile
     {
         const uint64_t table_tokens = (uint64_t)p.pages_per_request_layer << p.tokens_per_page_shift;
