@@ -35,9 +35,10 @@ inline uint64_t div_ceil_u64(uint64_t a, uint64_t b) { return a / b + (a % b != 
 
 inline bool is_power_of_two(uint32_t v) { return v != 0 && (v & (v - 1)) == 0; }
 
+// Smallest power of two >= v (2^31 for anything above it: the callers clamp long before that).
 inline uint32_t next_power_of_two(uint32_t v) {
     uint32_t p = 1;
-    while (p < v) p <<= 1;
+    while (p < v && p < 0x80000000u) p <<= 1;
     return p;
 }
 
