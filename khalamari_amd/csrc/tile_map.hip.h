@@ -123,7 +123,9 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         if (linear < main) work = (linear % 8) * per_xcd + linear / 8;
     }
     const uint32_t head_group = (uint32_t)(work / num_tasks);
-    const uint32_t task = (uint32_t)(work % num_tasks);
+    // Templates are taken last to first: within a request the later Q ranges see more keys, so the long blocks start
+    // early and the short ones fill the end of the launch (2 % on a batch of 2048-token chunks).
+    const uint32_t task = num_tasks - 1 - (uint32_t)(work % num_tasks);
 
     // ---- task decode (uniform) ---------------------------------------------------------------------------
     if (task >= resolve_u32(p.num_active_kv_splits, p.replay_parameters)) return;
