@@ -422,11 +422,12 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     // MFMAs depend on nothing the softmax produces, so the matrix pipe works on them while the VALU does the
     // exponentials (a software pipeline of depth one inside every wave).
     auto process_slice = [&](auto precise_tag, auto masked_tag, uint32_t slice_first, Scores& scores, const unsigned char* k_next,
-                             const unsigned char* v_src) __attribute__((always_inline)) {
+                             const unsigned char* v_src, auto&& behind_the_scores) __attribute__((always_inline)) {
         constexpr bool PRECISE = decltype(precise_tag)::value;
         constexpr bool MASKED = decltype(masked_tag)::value;
         Scores next;
         scores_of(k_next, next);
+        behind_the_scores();   // address arithmetic and load issue of a later tile, while the matrix pipe works on S^T
         uint32_t p_bits[NTW][4], p_low[PRECISE ? NTW : 1][4];
         f32x4 (&s)[2][NTW] = scores.s;
         // scores relative to the column reference, the lane's maximum, and whether any column must move
@@ -532,16 +533,23 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     };
     Scores pending;
     TileIds upcoming = fetch_ids(NSTAGES - 1);
+    // FP8 pages: decode tile + 2 from registers into LDS, request tile + 3.  The MFMA-bound tiles (two column tiles per
+    // wave) do it behind the first S^T of the tile like the bf16 path requests its loads (1.6 % on config 5); the
+    // bandwidth-bound verify tiles do it straight after the barrier, where the decoded tile is ready soonest (2 %).
+    constexpr bool kRawTileBehindScores = NTW >= 2;
+    auto advance_raw_tiles = [&](uint32_t tile) __attribute__((always_inline)) {
+        if (tile + 2 < num_tiles) write_raw_tile(tile + 2);
+        if (tile + 3 < num_tiles) {
+            load_raw_tile(tile + 3, upcoming);
+            upcoming = fetch_ids(tile + 4);
+        }
+    };
     auto run_tiles = [&](auto precise_tag, auto masked_tag, uint32_t tile_begin, uint32_t tile_end) __attribute__((always_inline)) {
         for (uint32_t tile = tile_begin; tile < tile_end; ++tile) {
             if constexpr (KV8) {
                 // tile + 1 was written to LDS during the previous tile; tile + 2 sits in registers, tile + 3 is requested
                 barrier_keeping_loads_in_flight();
-                if (tile + 2 < num_tiles) write_raw_tile(tile + 2);
-                if (tile + 3 < num_tiles) {
-                    load_raw_tile(tile + 3, upcoming);
-                    upcoming = fetch_ids(tile + 4);
-                }
+                if constexpr (!kRawTileBehindScores) advance_raw_tiles(tile);
             } else {
                 // at this point the loads of tiles up to tile + NSTAGES - 2 have been issued
                 if (tile + 1 < num_tiles) {
@@ -552,17 +560,27 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
                     else wait_vmem_outstanding<0>();
                 }
                 barrier_keeping_loads_in_flight();
-                if (tile + NSTAGES - 1 < num_tiles) {
-                    issue_tile(tile + NSTAGES - 1, upcoming);
-                    upcoming = fetch_ids(tile + NSTAGES);
-                }
             }
+            // The stage of tile - 1 is free from the barrier on; its next tenant is requested behind the first S^T of
+            // this tile rather than straight after the barrier, where all waves would do address arithmetic at once
+            // with the matrix pipe idle.
+            auto request_next = [&]() __attribute__((always_inline)) {
+                if constexpr (!KV8) {
+                    if (tile + NSTAGES - 1 < num_tiles) {
+                        issue_tile(tile + NSTAGES - 1, upcoming);
+                        upcoming = fetch_ids(tile + NSTAGES);
+                    }
+                }
+                if constexpr (KV8 && kRawTileBehindScores) advance_raw_tiles(tile);
+            };
+            auto nothing = []() __attribute__((always_inline)) {};
 #pragma unroll
             for (int k = 0; k < SL; ++k) {
                 const uint32_t slice = tile * SL + k;
                 if (k == 0 || slice < num_slices) {
                     const uint32_t following = slice + 1 < num_slices ? slice + 1 : slice;   // the last one recomputes itself, unused
-                    process_slice(precise_tag, masked_tag, first_token + slice * 32, pending, k_slice(following), v_slice(slice));
+                    if (k == 0) process_slice(precise_tag, masked_tag, first_token + slice * 32, pending, k_slice(following), v_slice(slice), request_next);
+                    else process_slice(precise_tag, masked_tag, first_token + slice * 32, pending, k_slice(following), v_slice(slice), nothing);
                 }
             }
         }
