@@ -507,7 +507,7 @@ def main() -> int:
     parser.add_argument("--producers", action="store_true",
                         help="time only the kernels that feed the SDPA (RMSNorm + RoPE, K/V page write) and print their JSON (profiling runs)")
     parser.add_argument("--fp8-pages", action="store_true",
-                        help="headline config on FP8 E4M3FN pages, the reference's cache format (profiling runs; the default headline is the bf16 pages BASELINE names)")
+                        help="headline config on FP8 E4M3FN pages, the reference's cache format (profiling runs; the default headline keeps bf16 pages)")
     parser.add_argument("--calibration-copy", action="store_true",
                         help="also launch a plain 1 GiB copy kernel, the known-size reference for FETCH_SIZE / WRITE_SIZE counter runs")
     args = parser.parse_args()
