@@ -31,12 +31,15 @@ class Workload:
 
 def make_workload(*, num_q_heads, num_kv_heads, head_dim, tokens_per_page, histories, q_lens, seed, scale=None,
                   num_layers=1, layer=0, page_ids_per_block=1, permute=True, spare_pages=3, value_scale=1.0,
-                  garbage_bits=None, req_slot_order=None, fp8_pages=False) -> Workload:
+                  garbage_bits=None, req_slot_order=None, fp8_pages=False, key_drift=None) -> Workload:
     """Sequences r = 0..R-1 with `histories[r]` cached tokens and `q_lens[r]` new Q tokens (already in the cache).
 
     K/V/Q ~ N(0, value_scale) rounded to bf16.  Pages come from one shared pool, randomly permuted.
     `garbage_bits`, when given, fills every unused page slot (tokens past a sequence's end) with that bf16
     pattern, e.g. 0x7fc0 (NaN), to prove masked slots never reach the output (an FP8 code with `fp8_pages`).
+    `key_drift` adds `key_drift * position` to dimension 0 of every key and sets dimension 0 of every query to 4: all
+    scores of a sequence rise steadily along the context, so they keep outgrowing whatever running maximum an online
+    softmax holds (its rescaling path runs many times) while the weights stay spread over many recent keys.
     `fp8_pages` stores K/V as FP8 E4M3FN codes; the values are quantised first, as the reference's tests do
     before their oracle sees them (sliced_kv_test.rs:484-493).
     """
@@ -58,7 +61,10 @@ def make_workload(*, num_q_heads, num_kv_heads, head_dim, tokens_per_page, histo
     cursor = 0
     for r in range(R):
         ctx = contexts[r]
-        k = oracle.bf16_round(rng.standard_normal((ctx, num_kv_heads, head_dim), dtype=np.float32) * value_scale)
+        k = rng.standard_normal((ctx, num_kv_heads, head_dim), dtype=np.float32) * value_scale
+        if key_drift is not None:
+            k[:, :, 0] += np.float32(key_drift) * np.arange(ctx, dtype=np.float32)[:, None]
+        k = oracle.bf16_round(k)
         v = oracle.bf16_round(rng.standard_normal((ctx, num_kv_heads, head_dim), dtype=np.float32) * value_scale)
         if fp8_pages:
             k, v = oracle.fp8_round_trip(k), oracle.fp8_round_trip(v)
@@ -71,6 +77,8 @@ def make_workload(*, num_q_heads, num_kv_heads, head_dim, tokens_per_page, histo
                                  fill_bits=0 if garbage_bits is None else garbage_bits)
     T = int(sum(q_lens))
     q = rng.standard_normal((T, num_q_heads, head_dim), dtype=np.float32) * value_scale
+    if key_drift is not None:
+        q[:, :, 0] = 4.0
     q_bits = oracle.f32_to_bf16_bits(q)
     req_slots = np.concatenate([np.full(n, slots[r], dtype=np.uint32) for r, n in enumerate(q_lens)])
     visible = np.zeros((T, 2), dtype=np.uint32)

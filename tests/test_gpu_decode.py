@@ -51,6 +51,12 @@ def test_unaligned_slices_and_nan_garbage(device):
     _decode_case(device, hq=16, hkv=2, d=128, tpp=16, histories=[130, 64, 7], kv_slice=65, seed=9, garbage_bits=0x7FC0)
 
 
+@pytest.mark.parametrize("d", [128, 256])
+def test_scores_that_keep_outgrowing_the_running_maximum(device, d):
+    """Scores rise steadily along the context: the online softmax has to rescale its accumulators again and again."""
+    _decode_case(device, hq=24, hkv=4, d=d, tpp=16, histories=[3000, 511, 40], kv_slice=1024, seed=77, key_drift=0.04)
+
+
 def test_fused_map_reduce_equals_two_launches(device):
     """One-launch Map+Reduce (the last block of a token merges) matches Map followed by Reduce to within one
     rounding of the merge order, and the oracle to the parity gate, also when launched repeatedly on the same
