@@ -384,9 +384,14 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     // the wave has to move.  lane_top[nt] is the largest score this lane has seen, relative to ref[nt]; the true
     // column maximum for the partial-state ABI is reduced across lanes once, in the epilogue.
     constexpr float kRescaleThreshold = 8.0f;
+    // Interior slices of a direct-output block: a lane whose eight weights add up to more than 2^8 has a score more than
+    // 5 above the reference; the reference then moves for every column whose maximum is more than 4 above it.
+    constexpr float kSumTrigger = 256.0f;
+    constexpr float kUntrackedMove = 4.0f;
     f32x4 acc[NTW][MT];
     float run_sum[NTW];
     float ref[NTW], lane_top[NTW];
+    bool unanchored = false;   // before an untracked run: this lane has a column tile without a visible key so far
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt) {
         ref[nt] = 0.0f;
@@ -421,76 +426,143 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     // One slice: softmax update of the pending S^T, then P.V.  The S^T of the following slice is computed first: its
     // MFMAs depend on nothing the softmax produces, so the matrix pipe works on them while the VALU does the
     // exponentials (a software pipeline of depth one inside every wave).
-    auto process_slice = [&](auto precise_tag, auto masked_tag, uint32_t slice_first, Scores& scores, const unsigned char* k_next,
-                             const unsigned char* v_src, auto&& behind_the_scores) __attribute__((always_inline)) {
+    auto process_slice = [&](auto precise_tag, auto masked_tag, auto untracked_tag, uint32_t slice_first, Scores& scores,
+                             const unsigned char* k_this, const unsigned char* k_next, const unsigned char* v_src, auto&& behind_the_scores) __attribute__((always_inline)) {
         constexpr bool PRECISE = decltype(precise_tag)::value;
         constexpr bool MASKED = decltype(masked_tag)::value;
+        // UNTRACKED: the largest score is not followed (direct output needs no partial state).  The weights are computed
+        // straight away and the lane's sum of them, which the slice needs anyway, tells whether a score ran away from
+        // the reference: one compare per column tile instead of a maximum over the lane's eight scores.
+        constexpr bool UNTRACKED = decltype(untracked_tag)::value;
+        static_assert(!UNTRACKED || (!PRECISE && !MASKED), "the untracked slice is the plain interior one");
         Scores next;
         scores_of(k_next, next);
         behind_the_scores();   // address arithmetic and load issue of a later tile, while the matrix pipe works on S^T
         uint32_t p_bits[NTW][4], p_low[PRECISE ? NTW : 1][4];
         f32x4 (&s)[2][NTW] = scores.s;
-        // scores relative to the column reference, the lane's maximum, and whether any column must move
-        float slice_top[NTW];
-        bool lane_wants_move = false;
+        if constexpr (UNTRACKED) {
+            float slice_sum[NTW];
+            auto weights = [&]() __attribute__((always_inline)) {
 #pragma unroll
-        for (int nt = 0; nt < NTW; ++nt) {
+                for (int nt = 0; nt < NTW; ++nt) {
+                    slice_sum[nt] = 0.0f;
 #pragma unroll
-            for (int rt = 0; rt < 2; ++rt)
+                    for (int rt = 0; rt < 2; ++rt) {
+                        float e[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    float value = __builtin_fmaf(s[rt][nt][i], p.scale_log2e, -ref[nt]);
-                    if constexpr (MASKED) {
-                        const uint32_t token = slice_first + rt * 16 + g * 4 + i;
-                        value = (token >= col_lo[nt] && token < col_hi[nt]) ? value : -INFINITY;
+                        for (int i = 0; i < 4; ++i) e[i] = fast_exp2(s[rt][nt][i]);
+                        slice_sum[nt] += (e[0] + e[1]) + (e[2] + e[3]);
+                        p_bits[nt][2 * rt] = pack_bf16x2(e[0], e[1]);
+                        p_bits[nt][2 * rt + 1] = pack_bf16x2(e[2], e[3]);
                     }
-                    s[rt][nt][i] = value;
                 }
-            slice_top[nt] = fmaxf(fmaxf(fmaxf(s[0][nt][0], s[0][nt][1]), fmaxf(s[0][nt][2], s[0][nt][3])),
-                                  fmaxf(fmaxf(s[1][nt][0], s[1][nt][1]), fmaxf(s[1][nt][2], s[1][nt][3])));
-            // a lane that has not seen a visible key yet cannot know whether its column has a reference
-            lane_wants_move = lane_wants_move | (slice_top[nt] > kRescaleThreshold) | (lane_top[nt] == -INFINITY);
-        }
-        if (__builtin_amdgcn_ballot_w64(lane_wants_move) != 0) {
-            // rare: agree per column (its four lanes) on the maximum, move the reference and rescale what was accumulated
+            };
+            bool lane_wants_move = unanchored;
+            auto relative_scores = [&]() __attribute__((always_inline)) {
 #pragma unroll
+                for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+                    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) s[rt][nt][i] = __builtin_fmaf(s[rt][nt][i], p.scale_log2e, -ref[nt]);
+            };
+            relative_scores();
+            weights();
+#pragma unroll
+            for (int nt = 0; nt < NTW; ++nt) lane_wants_move = lane_wants_move | !(slice_sum[nt] <= kSumTrigger);
+            if (__builtin_amdgcn_ballot_w64(lane_wants_move) != 0) {
+                // rare: some lane's weights add up to more than kSumTrigger (one of its scores is then more than
+                // kUntrackedMove above the reference), or a column has no reference yet.  The scores are computed again
+                // from the slice's keys, still in LDS, so that the common path need not keep them beyond the weights.
+                scores_of(k_this, scores);
+                relative_scores();
+#pragma unroll
+                for (int nt = 0; nt < NTW; ++nt) {
+                    const float lane_slice_top = fmaxf(fmaxf(fmaxf(s[0][nt][0], s[0][nt][1]), fmaxf(s[0][nt][2], s[0][nt][3])),
+                                                       fmaxf(fmaxf(s[1][nt][0], s[1][nt][1]), fmaxf(s[1][nt][2], s[1][nt][3])));
+                    const float column_top = max_over_rows(lane_slice_top);
+                    const bool first = max_over_rows(lane_top[nt]) == -INFINITY;
+                    const bool move = column_top > kUntrackedMove || first;   // every key of an interior slice is visible
+                    const float shift = move ? column_top : 0.0f;
+                    const float alpha = first ? 0.0f : fast_exp2(-shift);
+                    ref[nt] += shift;
+                    lane_top[nt] = fmaxf(lane_top[nt], lane_slice_top) - shift;   // only its finiteness is used from here on
+#pragma unroll
+                    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) s[rt][nt][i] -= shift;
+                    run_sum[nt] *= alpha;
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) acc[nt][mt] *= alpha;
+                }
+                weights();
+            }
+            unanchored = false;
+#pragma unroll
+            for (int nt = 0; nt < NTW; ++nt) run_sum[nt] += slice_sum[nt];
+        } else {
+            // scores relative to the column reference, the lane's maximum, and whether any column must move
+            float slice_top[NTW];
+            bool lane_wants_move = false;
+    #pragma unroll
             for (int nt = 0; nt < NTW; ++nt) {
-                const float column_top = max_over_rows(slice_top[nt]);
-                const float column_seen = max_over_rows(lane_top[nt]);
-                const bool first = column_seen == -INFINITY;
-                const bool move = column_top > kRescaleThreshold || (first && column_top > -INFINITY);
-                const float shift = move ? column_top : 0.0f;
-                const float alpha = first ? 0.0f : fast_exp2(-shift);   // nothing is accumulated before the first key
-                ref[nt] += shift;
-                lane_top[nt] -= shift;
-                slice_top[nt] -= shift;
-#pragma unroll
+    #pragma unroll
                 for (int rt = 0; rt < 2; ++rt)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) s[rt][nt][i] -= shift;
-                run_sum[nt] *= alpha;
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) acc[nt][mt] *= alpha;
+    #pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        float value = __builtin_fmaf(s[rt][nt][i], p.scale_log2e, -ref[nt]);
+                        if constexpr (MASKED) {
+                            const uint32_t token = slice_first + rt * 16 + g * 4 + i;
+                            value = (token >= col_lo[nt] && token < col_hi[nt]) ? value : -INFINITY;
+                        }
+                        s[rt][nt][i] = value;
+                    }
+                slice_top[nt] = fmaxf(fmaxf(fmaxf(s[0][nt][0], s[0][nt][1]), fmaxf(s[0][nt][2], s[0][nt][3])),
+                                      fmaxf(fmaxf(s[1][nt][0], s[1][nt][1]), fmaxf(s[1][nt][2], s[1][nt][3])));
+                // a lane that has not seen a visible key yet cannot know whether its column has a reference
+                lane_wants_move = lane_wants_move | (slice_top[nt] > kRescaleThreshold) | (lane_top[nt] == -INFINITY);
             }
-        }
-#pragma unroll
-        for (int nt = 0; nt < NTW; ++nt) {
-            lane_top[nt] = fmaxf(lane_top[nt], slice_top[nt]);
-            float slice_sum = 0.0f;
-#pragma unroll
-            for (int rt = 0; rt < 2; ++rt) {
-                float e[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) e[i] = fast_exp2(s[rt][nt][i]);
-                slice_sum += (e[0] + e[1]) + (e[2] + e[3]);
-                p_bits[nt][2 * rt] = pack_bf16x2(e[0], e[1]);
-                p_bits[nt][2 * rt + 1] = pack_bf16x2(e[2], e[3]);
-                if constexpr (PRECISE) {
-                    p_low[nt][2 * rt] = pack_bf16x2(e[0] - bf16_bits_to_f32(p_bits[nt][2 * rt] & 0xffffu), e[1] - bf16_bits_to_f32(p_bits[nt][2 * rt] >> 16));
-                    p_low[nt][2 * rt + 1] = pack_bf16x2(e[2] - bf16_bits_to_f32(p_bits[nt][2 * rt + 1] & 0xffffu), e[3] - bf16_bits_to_f32(p_bits[nt][2 * rt + 1] >> 16));
+            if (__builtin_amdgcn_ballot_w64(lane_wants_move) != 0) {
+                // rare: agree per column (its four lanes) on the maximum, move the reference and rescale what was accumulated
+    #pragma unroll
+                for (int nt = 0; nt < NTW; ++nt) {
+                    const float column_top = max_over_rows(slice_top[nt]);
+                    const float column_seen = max_over_rows(lane_top[nt]);
+                    const bool first = column_seen == -INFINITY;
+                    const bool move = column_top > kRescaleThreshold || (first && column_top > -INFINITY);
+                    const float shift = move ? column_top : 0.0f;
+                    const float alpha = first ? 0.0f : fast_exp2(-shift);   // nothing is accumulated before the first key
+                    ref[nt] += shift;
+                    lane_top[nt] -= shift;
+                    slice_top[nt] -= shift;
+    #pragma unroll
+                    for (int rt = 0; rt < 2; ++rt)
+    #pragma unroll
+                        for (int i = 0; i < 4; ++i) s[rt][nt][i] -= shift;
+                    run_sum[nt] *= alpha;
+    #pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) acc[nt][mt] *= alpha;
                 }
             }
-            run_sum[nt] += slice_sum;
+    #pragma unroll
+            for (int nt = 0; nt < NTW; ++nt) {
+                lane_top[nt] = fmaxf(lane_top[nt], slice_top[nt]);
+                float slice_sum = 0.0f;
+    #pragma unroll
+                for (int rt = 0; rt < 2; ++rt) {
+                    float e[4];
+    #pragma unroll
+                    for (int i = 0; i < 4; ++i) e[i] = fast_exp2(s[rt][nt][i]);
+                    slice_sum += (e[0] + e[1]) + (e[2] + e[3]);
+                    p_bits[nt][2 * rt] = pack_bf16x2(e[0], e[1]);
+                    p_bits[nt][2 * rt + 1] = pack_bf16x2(e[2], e[3]);
+                    if constexpr (PRECISE) {
+                        p_low[nt][2 * rt] = pack_bf16x2(e[0] - bf16_bits_to_f32(p_bits[nt][2 * rt] & 0xffffu), e[1] - bf16_bits_to_f32(p_bits[nt][2 * rt] >> 16));
+                        p_low[nt][2 * rt + 1] = pack_bf16x2(e[2] - bf16_bits_to_f32(p_bits[nt][2 * rt + 1] & 0xffffu), e[3] - bf16_bits_to_f32(p_bits[nt][2 * rt + 1] >> 16));
+                    }
+                }
+                run_sum[nt] += slice_sum;
+            }
         }
         // O^T += V^T . P^T over the 32 tokens: k = 8g + j <-> token (j < 4 ? 4g + j : 16 + 4g + j - 4) of the slice.
 #pragma unroll
@@ -544,7 +616,7 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             upcoming = fetch_ids(tile + 4);
         }
     };
-    auto run_tiles = [&](auto precise_tag, auto masked_tag, uint32_t tile_begin, uint32_t tile_end) __attribute__((always_inline)) {
+    auto run_tiles = [&](auto precise_tag, auto masked_tag, auto untracked_tag, uint32_t tile_begin, uint32_t tile_end) __attribute__((always_inline)) {
         for (uint32_t tile = tile_begin; tile < tile_end; ++tile) {
             if constexpr (KV8) {
                 // tile + 1 was written to LDS during the previous tile; tile + 2 sits in registers, tile + 3 is requested
@@ -579,8 +651,8 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
                 const uint32_t slice = tile * SL + k;
                 if (k == 0 || slice < num_slices) {
                     const uint32_t following = slice + 1 < num_slices ? slice + 1 : slice;   // the last one recomputes itself, unused
-                    if (k == 0) process_slice(precise_tag, masked_tag, first_token + slice * 32, pending, k_slice(following), v_slice(slice), request_next);
-                    else process_slice(precise_tag, masked_tag, first_token + slice * 32, pending, k_slice(following), v_slice(slice), nothing);
+                    if (k == 0) process_slice(precise_tag, masked_tag, untracked_tag, first_token + slice * 32, pending, k_slice(slice), k_slice(following), v_slice(slice), request_next);
+                    else process_slice(precise_tag, masked_tag, untracked_tag, first_token + slice * 32, pending, k_slice(slice), k_slice(following), v_slice(slice), nothing);
                 }
             }
         }
@@ -610,14 +682,27 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         uint32_t tail_begin = wave_all_hi > first_token ? (wave_all_hi - first_token) / BK : 0;
         tail_begin = tail_begin < num_tiles ? tail_begin : num_tiles;
         tail_begin = tail_begin > head_end ? tail_begin : head_end;
+        constexpr std::true_type yes{};
+        constexpr std::false_type no{};
         if (precise) {
-            run_tiles(std::true_type{}, std::true_type{}, 0, head_end);
-            run_tiles(std::true_type{}, std::false_type{}, head_end, tail_begin);
-            run_tiles(std::true_type{}, std::true_type{}, tail_begin, num_tiles);
+            run_tiles(yes, yes, no, 0, head_end);
+            run_tiles(yes, no, no, head_end, tail_begin);
+            run_tiles(yes, yes, no, tail_begin, num_tiles);
         } else {
-            run_tiles(std::false_type{}, std::true_type{}, 0, head_end);
-            run_tiles(std::false_type{}, std::false_type{}, head_end, tail_begin);
-            run_tiles(std::false_type{}, std::true_type{}, tail_begin, num_tiles);
+            run_tiles(no, yes, no, 0, head_end);
+            // The extra loop pays where the tile is bound by instruction issue and has registers to spare: two column
+            // tiles per wave at D 128 on bf16 pages (FP8 pages keep a raw tile in registers, D 256 twice the
+            // accumulators; there the spills cost more than the maxima saved).
+            constexpr bool kUntrackedInterior = !KV8 && NTW >= 2 && D == 128;
+            if (kUntrackedInterior && p.output_mode == kMapDirectBf16) {
+                // no partial state to hand on: the interior slices need not follow the largest score
+#pragma unroll
+                for (int nt = 0; nt < NTW; ++nt) unanchored = unanchored | (lane_top[nt] == -INFINITY);
+                run_tiles(no, no, yes, head_end, tail_begin);
+            } else {
+                run_tiles(no, no, no, head_end, tail_begin);
+            }
+            run_tiles(no, yes, no, tail_begin, num_tiles);
         }
     }
 
