@@ -690,10 +690,11 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             run_tiles(yes, yes, no, tail_begin, num_tiles);
         } else {
             run_tiles(no, yes, no, 0, head_end);
-            // The extra loop pays where the tile is bound by instruction issue and has registers to spare: two column
-            // tiles per wave at D 128 on bf16 pages (FP8 pages keep a raw tile in registers, D 256 twice the
-            // accumulators; there the spills cost more than the maxima saved).
-            constexpr bool kUntrackedInterior = !KV8 && NTW >= 2 && D == 128;
+            // The extra loop pays where the tile is bound by instruction issue and has registers to spare: the 256-column
+            // tile at D 128 on bf16 pages.  FP8 pages keep a raw tile in registers, D 256 has twice the accumulators and
+            // the 128-column tile runs two blocks per compute unit: there the spills cost more than the maxima saved
+            // (the 128-column tile on the prefill benchmark: 6.9 ms without, 10 ms with).
+            constexpr bool kUntrackedInterior = !KV8 && NTW >= 2 && NWAVES == 8 && D == 128;
             if (kUntrackedInterior && p.output_mode == kMapDirectBf16) {
                 // no partial state to hand on: the interior slices need not follow the largest score
 #pragma unroll
