@@ -52,7 +52,19 @@ struct TileKernelChoice {
 
 // Tiled (LDS-shared K/V) kernel for Q tiles of 17..256 coordinates: speculative-verify blocks (one 16-column tile per
 // wave, bandwidth-bound) up to prefill tiles (32 columns per wave, MFMA-bound).
-static TileKernelChoice select_tile_kernel(uint32_t head_dim, uint32_t coordinates, uint32_t kv_dtype) {
+static TileKernelChoice select_tile_kernel(uint32_t head_dim, uint32_t coordinates, uint32_t kv_dtype, bool direct) {
+    // The MFMA-bound tiles (two column tiles per wave) at D 128 have a build of their own for computes that only ever
+    // write final output: its interior slices do not follow the largest score.  (One kernel holding both kinds of
+    // interior loop spills; the one-column-tile and D 256 tiles gain nothing from it.)
+    if (direct && head_dim == 128 && coordinates > 64) {
+        const bool wide = coordinates > 128;
+        if (kv_dtype == KHM_DTYPE_FP8_E4M3FN) {
+            if (wide) return {tile_map_kernel<128, 2, 8, 64, 4, 1, true, true>, 512, (uint32_t)TileSmem<128, 64, 4>::kBytes};
+            return {tile_map_kernel<128, 2, 4, 64, 4, 2, true, true>, 256, (uint32_t)TileSmem<128, 64, 4>::kBytes};
+        }
+        if (wide) return {tile_map_kernel<128, 2, 8, 64, 4, 1, false, true>, 512, (uint32_t)TileSmem<128, 64, 4>::kBytes};
+        return {tile_map_kernel<128, 2, 4, 64, 4, 2, false, true>, 256, (uint32_t)TileSmem<128, 64, 4>::kBytes};
+    }
     if (kv_dtype == KHM_DTYPE_FP8_E4M3FN) {
         if (head_dim == 128) {
             if (coordinates <= 64) return {tile_map_kernel<128, 1, 4, 32, 4, 2, true>, 256, (uint32_t)TileSmem<128, 32, 4>::kBytes};
@@ -477,7 +489,7 @@ extern "C" int khm_sliced_q_create(const khm_gqa_sdpa_config* config, const khm_
         compute->map_merges_in_kernel = true;
     } else {
         compute->map_merges_in_kernel = false;
-        const TileKernelChoice choice = select_tile_kernel(config->head_dim, coordinates, config->kv_dtype);
+        const TileKernelChoice choice = select_tile_kernel(config->head_dim, coordinates, config->kv_dtype, compute->direct);
         compute->map = choice.kernel;
         compute->map_threads = choice.threads;
         compute->map_smem_bytes = choice.smem_bytes;

@@ -80,7 +80,9 @@ __device__ __forceinline__ uint32_t load_uniform_u32(const uint32_t* table, uint
 // load is unchanged; the tile itself travels through registers (16 bytes = 16 codes per lane and load), is decoded
 // there and written to LDS one barrier before it is first read.  One tile is in flight in registers while two are
 // consumed: enough for the MFMA-bound prefill tiles this mode is built for.
-template <int D, int NTW, int NWAVES, int BK, int NSTAGES, int MIN_BLOCKS, bool KV8 = false>
+// DIRECT: the instantiation only ever writes final output (p.output_mode == kMapDirectBf16, which the host guarantees);
+// it exists where following the largest score is worth compiling out, see the untracked slices below.
+template <int D, int NTW, int NWAVES, int BK, int NSTAGES, int MIN_BLOCKS, bool KV8 = false, bool DIRECT = false>
 __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const MapParams p) {
     constexpr int KS = D / 32;                      // QK k-steps
     constexpr int MT = D / 16;                      // PV dim tiles
@@ -690,12 +692,7 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             run_tiles(yes, yes, no, tail_begin, num_tiles);
         } else {
             run_tiles(no, yes, no, 0, head_end);
-            // The extra loop pays where the tile is bound by instruction issue and has registers to spare: the 256-column
-            // tile at D 128 on bf16 pages.  FP8 pages keep a raw tile in registers, D 256 has twice the accumulators and
-            // the 128-column tile runs two blocks per compute unit: there the spills cost more than the maxima saved
-            // (the 128-column tile on the prefill benchmark: 6.9 ms without, 10 ms with).
-            constexpr bool kUntrackedInterior = !KV8 && NTW >= 2 && NWAVES == 8 && D == 128;
-            if (kUntrackedInterior && p.output_mode == kMapDirectBf16) {
+            if constexpr (DIRECT) {
                 // no partial state to hand on: the interior slices need not follow the largest score
 #pragma unroll
                 for (int nt = 0; nt < NTW; ++nt) unanchored = unanchored | (lane_top[nt] == -INFINITY);
@@ -708,7 +705,7 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     }
 
     // ---- epilogue: every wave owns its columns, no cross-wave merge ------------------------------------------------
-    const uint32_t mode = p.output_mode;
+    const uint32_t mode = DIRECT ? (uint32_t)kMapDirectBf16 : p.output_mode;
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt) {
         // the lanes of a column each hold the sum over their tokens, relative to ref[nt]

@@ -350,21 +350,27 @@ def test_chunked_prefill_onto_a_paged_prefix(device, hq, hkv, d, tile):
         helpers.assert_parity(actual, expected, f"prefill tile={tile} slice={kv_slice} direct={direct}")
 
 
-@pytest.mark.parametrize("hq,hkv,d,tile", [(64, 8, 128, 32), (32, 8, 128, 4), (24, 4, 256, 16)])
-def test_scores_that_keep_outgrowing_the_running_reference(device, hq, hkv, d, tile):
+@pytest.mark.parametrize("hq,hkv,d,tile,fp8", [(64, 8, 128, 32, False), (64, 8, 128, 16, False), (64, 8, 128, 32, True),
+                                               (32, 4, 128, 16, True), (32, 8, 128, 4, False), (24, 4, 256, 16, False)])
+def test_scores_that_keep_outgrowing_the_running_reference(device, hq, hkv, d, tile, fp8):
     """Every score of a sequence rises steadily along the context (by some 60 octaves over 3000 keys), so later scores
-    exceed the earlier maximum by far more than any rescaling threshold, over and over: the reference-moving path of the tiles runs many times, in the masked head and
-    tail tiles and in the interior ones, with direct output (which does not follow the largest score) and with
-    partial states + Reduce (which must report it)."""
+    exceed the earlier maximum by far more than any rescaling threshold, over and over: the reference-moving path of
+    the tiles runs many times, in the masked head and tail tiles and in the interior ones, with direct output (whose
+    two-column-tile builds at D 128 do not follow the largest score) and with partial states + Reduce (which must
+    report it), on bf16 and FP8 pages."""
     histories = [0, 700, 2500]
     q_lens = [96, 64, 40]
     w = helpers.make_workload(num_q_heads=hq, num_kv_heads=hkv, head_dim=d, tokens_per_page=16, histories=histories,
-                              q_lens=q_lens, seed=300 + tile, key_drift=0.04)
+                              q_lens=q_lens, seed=300 + tile, key_drift=0.04, fp8_pages=fp8)
     expected = helpers.expected_output(w)
     ratio = hq // hkv
     for kv_slice, direct in [(1 << 20, True), (1024, False)]:
         ranges, templates, cu = helpers.fixed_slice_plan(histories, q_lens, tile, kv_slice)
-        print(f"growing scores hq={hq} hkv={hkv} d={d} tile={tile} kv_slice={kv_slice} direct={direct}", flush=True)
+        print(f"growing scores hq={hq} hkv={hkv} d={d} tile={tile} fp8={fp8} kv_slice={kv_slice} direct={direct}", flush=True)
         actual = gpu_runner.run_sliced_q(w, ranges, templates, cu, device, kind=sdpa.MAP_Q_TOKENS_AND_HEADS, max_q_tokens=tile,
                                          max_q_heads=ratio, stage=64, direct=direct)
-        helpers.assert_parity(actual, expected, f"growing scores tile={tile} slice={kv_slice} direct={direct}")
+        # On FP8 pages the drifting key dimension climbs in steps of an eighth of its value, so the weights pile up on the
+        # few keys behind the latest step; single-rounded bf16 weights then show at 2-5e-3 on outputs of order one.  Still
+        # four times tighter than the reference's own component tests (2e-2 per element, sliced_kv_test.rs:183,511-530).
+        helpers.assert_parity(actual, expected, f"growing scores tile={tile} slice={kv_slice} direct={direct}",
+                              abs_tol=5.0e-3 if fp8 else helpers.ABS_TOL)
