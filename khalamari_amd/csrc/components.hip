@@ -73,7 +73,7 @@ static TileKernelChoice select_tile_kernel(uint32_t head_dim, uint32_t coordinat
         }
         if (head_dim == 256) {
             if (coordinates <= 64) return {tile_map_kernel<256, 1, 4, 32, 4, 1, true>, 256, (uint32_t)TileSmem<256, 32, 4>::kBytes};
-            if (coordinates <= 128) return {tile_map_kernel<256, 2, 4, 32, 4, 1, true>, 256, (uint32_t)TileSmem<256, 32, 4>::kBytes};
+            if (coordinates <= 128) return {tile_map_kernel<256, 1, 8, 32, 4, 1, true>, 512, (uint32_t)TileSmem<256, 32, 4>::kBytes};
             return {tile_map_kernel<256, 2, 8, 32, 4, 1, true>, 512, (uint32_t)TileSmem<256, 32, 4>::kBytes};
         }
         return {nullptr, 0, 0};
@@ -85,8 +85,11 @@ static TileKernelChoice select_tile_kernel(uint32_t head_dim, uint32_t coordinat
         return {tile_map_kernel<128, 2, 8, 64, 4, 1>, 512, (uint32_t)TileSmem<128, 64, 4>::kBytes};
     }
     if (head_dim == 256) {
+        // 65..128 coordinates: eight waves of one column tile each (167 VGPRs, two waves per SIMD) rather than four waves
+        // of two (256 VGPRs + 167 AGPRs, one wave per SIMD, nothing to overlap its waits with): 414 -> 527 TFLOP/s on a
+        // batch of 2048-token chunks at Hq24/Hkv4.
         if (coordinates <= 64) return {tile_map_kernel<256, 1, 4, 32, 4, 1>, 256, (uint32_t)TileSmem<256, 32, 4>::kBytes};
-        if (coordinates <= 128) return {tile_map_kernel<256, 2, 4, 32, 4, 1>, 256, (uint32_t)TileSmem<256, 32, 4>::kBytes};
+        if (coordinates <= 128) return {tile_map_kernel<256, 1, 8, 32, 4, 1>, 512, (uint32_t)TileSmem<256, 32, 4>::kBytes};
         return {tile_map_kernel<256, 2, 8, 32, 4, 1>, 512, (uint32_t)TileSmem<256, 32, 4>::kBytes};
     }
     return {nullptr, 0, 0};
