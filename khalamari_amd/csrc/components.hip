@@ -53,9 +53,15 @@ struct TileKernelChoice {
 // Tiled (LDS-shared K/V) kernel for Q tiles of 17..256 coordinates: speculative-verify blocks (one 16-column tile per
 // wave, bandwidth-bound) up to prefill tiles (32 columns per wave, MFMA-bound).
 static TileKernelChoice select_tile_kernel(uint32_t head_dim, uint32_t coordinates, uint32_t kv_dtype, bool direct) {
-    // The MFMA-bound tiles (two column tiles per wave) at D 128 have a build of their own for computes that only ever
-    // write final output: its interior slices do not follow the largest score.  (One kernel holding both kinds of
-    // interior loop spills; the one-column-tile and D 256 tiles gain nothing from it.)
+    // The MFMA-bound tiles have a build of their own for computes that only ever write final output: its interior slices
+    // do not follow the largest score.  (One kernel holding both kinds of interior loop spills.)  These are the two-
+    // column-tile kernels at D 128 and the eight-wave tile at D 256 (523 -> 638 TFLOP/s on 2048-token chunks at
+    // Hq24/Hkv4); the bandwidth-bound verify tiles have nothing to gain.
+    if (direct && head_dim == 256 && coordinates > 64 && coordinates <= 128) {
+        if (kv_dtype == KHM_DTYPE_FP8_E4M3FN)
+            return {tile_map_kernel<256, 1, 8, 32, 4, 1, true, true>, 512, (uint32_t)TileSmem<256, 32, 4>::kBytes};
+        return {tile_map_kernel<256, 1, 8, 32, 4, 1, false, true>, 512, (uint32_t)TileSmem<256, 32, 4>::kBytes};
+    }
     if (direct && head_dim == 128 && coordinates > 64) {
         const bool wide = coordinates > 128;
         if (kv_dtype == KHM_DTYPE_FP8_E4M3FN) {

@@ -351,7 +351,8 @@ def test_chunked_prefill_onto_a_paged_prefix(device, hq, hkv, d, tile):
 
 
 @pytest.mark.parametrize("hq,hkv,d,tile,fp8", [(64, 8, 128, 32, False), (64, 8, 128, 16, False), (64, 8, 128, 32, True),
-                                               (32, 4, 128, 16, True), (32, 8, 128, 4, False), (24, 4, 256, 16, False)])
+                                               (32, 4, 128, 16, True), (32, 8, 128, 4, False), (24, 4, 256, 16, False),
+                                               (24, 4, 256, 16, True)])
 def test_scores_that_keep_outgrowing_the_running_reference(device, hq, hkv, d, tile, fp8):
     """Every score of a sequence rises steadily along the context (by some 60 octaves over 3000 keys), so later scores
     exceed the earlier maximum by far more than any rescaling threshold, over and over: the reference-moving path of
