@@ -44,10 +44,21 @@ CONFIGS = {
     5: dict(name="config5: B=8 chunked prefill, 2048-token chunk on prefix U[0,16384], Hq64/Hkv8/D128", hq=64, hkv=8, d=128,
             kind="prefill"),
 }
+# Not a benchmark config: the lengths of config 5 on the head geometry of config 3, so that the D 256 prefill tiles
+# have a measured figure too.  Reported under "configs" as "extra_prefill_d256"; selectable with --config 6.
+EXTRA_PREFILL_D256 = 6
+CONFIGS[EXTRA_PREFILL_D256] = dict(name="extra: B=8 chunked prefill, 2048-token chunk on prefix U[0,16384], Hq24/Hkv4/D256",
+                                   hq=24, hkv=4, d=256, kind="prefill")
+
+
+def config_key(index: int) -> str:
+    return "extra_prefill_d256" if index == EXTRA_PREFILL_D256 else f"config{index}"
 
 
 def sample_lengths(index: int):
     """(histories, q_lens) of a config; numpy PCG64 seeded with the config index."""
+    if index == EXTRA_PREFILL_D256:
+        return sample_lengths(5)
     rng = np.random.default_rng(index)
     if index == 1:
         return [1023], [1]
@@ -537,11 +548,11 @@ def main() -> int:
                 continue
             try:
                 workload = Workload(index, device)
-                others[f"config{index}"] = workload.report(max(args.steps // 4, 10), max(args.warmup // 2, 3))
+                others[config_key(index)] = workload.report(max(args.steps // 4, 10), max(args.warmup // 2, 3))
                 del workload
                 torch.cuda.empty_cache()
             except Exception as error:  # a config whose kernel is not built yet is reported, not hidden
-                others[f"config{index}"] = {"workload": CONFIGS[index]["name"], "error": str(error)}
+                others[config_key(index)] = {"workload": CONFIGS[index]["name"], "error": str(error)}
         # the reference's production cache format: half the bytes per KV token
         for index in (2, 3, 4, 5):
             try:
