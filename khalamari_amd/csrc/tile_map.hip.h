@@ -194,6 +194,13 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         other = __shfl_xor(wave_all_hi, offset); wave_all_hi = other < wave_all_hi ? other : wave_all_hi;
         other = __shfl_xor(min_span, offset); min_span = other < min_span ? other : min_span;
     }
+    // A wave none of whose columns is active (a request with fewer Q tokens than the tile has slots, fewer Q heads than
+    // the tile has columns for) still loads its share of every K/V tile and meets every barrier, but computes nothing:
+    // its LDS reads and matrix instructions would only take issue slots from the waves it shares a SIMD with.
+    bool lane_has_column = false;
+#pragma unroll
+    for (int nt = 0; nt < NTW; ++nt) lane_has_column = lane_has_column | col_active[nt];
+    const bool wave_idle = __builtin_amdgcn_ballot_w64(lane_has_column) == 0;
     // a slice is "interior" for the wave when every active column of the wave sees all of its 32 tokens
     wave_all_lo = __builtin_amdgcn_readfirstlane(wave_all_lo);
     wave_all_hi = __builtin_amdgcn_readfirstlane(wave_all_hi);
@@ -677,6 +684,29 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             wait_for_tile(0);
         }
         barrier_keeping_loads_in_flight();
+        if (wave_idle) {
+            // the loads, waits and barriers of run_tiles, nothing else
+            for (uint32_t tile = 0; tile < num_tiles; ++tile) {
+                if constexpr (KV8) {
+                    barrier_keeping_loads_in_flight();
+                    advance_raw_tiles(tile);
+                } else {
+                    if (tile + 1 < num_tiles) {
+                        const uint32_t last_issued = tile + NSTAGES - 2 < num_tiles - 1 ? tile + NSTAGES - 2 : num_tiles - 1;
+                        const uint32_t newer = last_issued - (tile + 1);
+                        if (NSTAGES >= 5 && newer >= 2) wait_vmem_outstanding<2 * LPW>();
+                        else if (newer >= 1) wait_vmem_outstanding<LPW>();
+                        else wait_vmem_outstanding<0>();
+                    }
+                    barrier_keeping_loads_in_flight();
+                    if (tile + NSTAGES - 1 < num_tiles) {
+                        issue_tile(tile + NSTAGES - 1, upcoming);
+                        upcoming = fetch_ids(tile + NSTAGES);
+                    }
+                }
+            }
+            return;   // no column of this wave is stored
+        }
         scores_of(k_slice(0), pending);
         // tiles [0, head_end) and [tail_begin, num_tiles) hold tokens some active column of the wave does not see
         uint32_t head_end = wave_all_lo > first_token ? (wave_all_lo - first_token + BK - 1) / BK : 0;
