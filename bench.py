@@ -51,6 +51,38 @@ CONFIGS[EXTRA_PREFILL_D256] = dict(name="extra: B=8 chunked prefill, 2048-token 
                                    hq=24, hkv=4, d=256, kind="prefill")
 
 
+SLAB_BYTES = 4096
+_slab_reader_lib = None
+
+
+def slab_read(pool, slab_ids, num_slabs: int, sink, blocks_per_cu: int = 2) -> None:
+    """Enqueues, on torch's current stream, a launch that only reads `num_slabs` slabs of 4096 bytes of `pool` (slab i at
+    byte offset `slab_ids[i] * 4096`) from a resident grid, in the Map kernel's lane layout.  The kernel lives in
+    `libbench_slab_read.so` beside this file (source `bench_slab_read.hip`): a measurement aid, not part of the library."""
+    import ctypes
+
+    import torch
+
+    global _slab_reader_lib
+    if _slab_reader_lib is None:
+        path = os.path.join(ROOT, "libbench_slab_read.so")
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is missing: run `python -m khalamari_amd.build` (or __graft_entry__.build()) first")
+        _slab_reader_lib = ctypes.CDLL(path)
+        _slab_reader_lib.bench_slab_read.restype = ctypes.c_int
+        _slab_reader_lib.bench_slab_read.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint32,
+                                                     ctypes.c_uint32, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
+
+    def nbytes(t):
+        return t.numel() * t.element_size()
+
+    status = _slab_reader_lib.bench_slab_read(pool.data_ptr(), nbytes(pool), slab_ids.data_ptr(), nbytes(slab_ids), int(num_slabs),
+                                              int(blocks_per_cu), sink.data_ptr(), nbytes(sink),
+                                              ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    if status != 0:
+        raise RuntimeError(f"bench_slab_read failed with status {status}")
+
+
 def config_key(index: int) -> str:
     return "extra_prefill_d256" if index == EXTRA_PREFILL_D256 else f"config{index}"
 
@@ -307,29 +339,27 @@ class Workload:
         with every wave the same share.  No metadata chain, no softmax, no merge, no ragged tail."""
         import torch
 
-        from khalamari_amd import calibration
-
         spec = self.spec
         kv_bytes = self.visible_tokens * spec["hkv"] * spec["d"] * 2 * self.kv_element_bytes
-        pool_slabs = self.kv_pools[0].numel() * self.kv_pools[0].element_size() // calibration.SLAB_BYTES
-        num_slabs = min(kv_bytes // calibration.SLAB_BYTES, pool_slabs)
+        pool_slabs = self.kv_pools[0].numel() * self.kv_pools[0].element_size() // SLAB_BYTES
+        num_slabs = min(kv_bytes // SLAB_BYTES, pool_slabs)
         order = np.random.Generator(np.random.PCG64(1234)).permutation(pool_slabs)[:num_slabs].astype(np.uint32)
         slab_ids = torch.from_numpy(order.view(np.int32)).to(self.kv_pools[0].device)
         sink = torch.zeros(1, dtype=torch.int32, device=slab_ids.device)
         best = None
         for blocks_per_cu in (2, 4):
             for i in range(3):
-                calibration.slab_read(self.kv_pools[i % len(self.kv_pools)], slab_ids, num_slabs, sink, blocks_per_cu)
+                slab_read(self.kv_pools[i % len(self.kv_pools)], slab_ids, num_slabs, sink, blocks_per_cu)
             pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
             for i, (a, b) in enumerate(pairs):
                 a.record()
-                calibration.slab_read(self.kv_pools[i % len(self.kv_pools)], slab_ids, num_slabs, sink, blocks_per_cu)
+                slab_read(self.kv_pools[i % len(self.kv_pools)], slab_ids, num_slabs, sink, blocks_per_cu)
                 b.record()
             torch.cuda.synchronize()
             mean_us = float(np.mean([a.elapsed_time(b) for a, b in pairs])) * 1e3
             if best is None or mean_us < best["us"]:
                 best = {"us": mean_us, "blocks_per_cu": blocks_per_cu}
-        nbytes = num_slabs * calibration.SLAB_BYTES
+        nbytes = num_slabs * SLAB_BYTES
         best.update(bytes=int(nbytes), gbps=nbytes / (best["us"] * 1e-6) / 1e9,
                     what="read-only launch of the workload's K/V bytes as random 4 KB slabs of the same pools, evenly split over a resident grid")
         return best

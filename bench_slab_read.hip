@@ -1,14 +1,12 @@
-// Measurement aid, not part of the attention path: a kernel that only reads a list of 4 KB slabs of a K/V pool, in
-// the lane layout and with the two tiles in flight per wave that the split-KV Map kernel uses, from a resident grid
-// whose waves all get the same number of slabs.  It does no arithmetic worth the name, has no dependent metadata
+// Measurement aid of bench.py, not part of the attention library (it is built into a library of its own, beside
+// bench.py): a kernel that only reads a list of 4 KB slabs of a K/V pool, in the lane layout and with the two tiles in
+// flight per wave that the split-KV Map kernel uses, from a resident grid whose waves all get the same number of slabs.  It does no arithmetic worth the name, has no dependent metadata
 // loads, no merge and no imbalance, so its time for N bytes is what this memory system gives a launch of that size
 // and access pattern; the benchmark reports it beside the Map kernel's time for the same bytes.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include "common.h"
-
-namespace khm {
+namespace {
 
 constexpr uint32_t kSlabBytes = 4096;   // 16 token rows of one KV head at head_dim 128, bf16
 
@@ -44,27 +42,21 @@ __global__ __launch_bounds__(256) void calibration_slab_read_kernel(const unsign
     if (folded == 0x9e3779b9u) sink[0] = folded;   // keeps the loads alive; practically never taken
 }
 
-}  // namespace khm
+}  // namespace
 
-using namespace khm;
-
-extern "C" int khm_calibration_slab_read(khm_buffer pool, khm_buffer slab_ids, uint32_t num_slabs, uint32_t blocks_per_cu, khm_buffer sink,
-                                         void* stream) {
-    clear_error();
-    KHM_REQUIRE(pool.ptr != nullptr && slab_ids.ptr != nullptr && sink.ptr != nullptr, "pool, slab_ids and sink must not be null");
-    KHM_REQUIRE(num_slabs > 0 && (uint64_t)num_slabs * 4 <= slab_ids.len_bytes, "slab_ids holds fewer than num_slabs entries");
-    KHM_REQUIRE(sink.len_bytes >= 4, "sink needs four bytes");
-    KHM_REQUIRE(blocks_per_cu >= 1 && blocks_per_cu <= 8, "blocks_per_cu must be 1..8");
-    KHM_REQUIRE(pool.len_bytes >= kSlabBytes && pool.len_bytes / kSlabBytes <= 0xffffffffull, "pool must hold 1 .. 2^32-1 slabs of 4096 bytes");
+// Returns 0, or 1 for a bad argument, 2 for a HIP error (the launch is enqueued on `stream`, never synchronized).
+extern "C" int bench_slab_read(const void* pool, uint64_t pool_bytes, const uint32_t* slab_ids, uint64_t slab_ids_bytes, uint32_t num_slabs,
+                               uint32_t blocks_per_cu, uint32_t* sink, uint64_t sink_bytes, void* stream) {
+    if (pool == nullptr || slab_ids == nullptr || sink == nullptr) return 1;
+    if (num_slabs == 0 || (uint64_t)num_slabs * 4 > slab_ids_bytes) return 1;
+    if (sink_bytes < 4 || blocks_per_cu < 1 || blocks_per_cu > 8) return 1;
+    if (pool_bytes < kSlabBytes || pool_bytes / kSlabBytes > 0xffffffffull) return 1;
     int device = 0, compute_units = 0;
     hipError_t status = hipGetDevice(&device);
     if (status == hipSuccess) status = hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device);
-    if (status != hipSuccess || compute_units <= 0) return fail(KHM_ERR_HIP, "could not read the compute unit count: %s", hipGetErrorString(status));
-    // The slab ids are the caller's and are not read back here: ids beyond the pool are the caller's bug, as with page ids.
+    if (status != hipSuccess || compute_units <= 0) return 2;
+    // The slab ids are the caller's and are not read back here: ids beyond the pool are the caller's bug.
     hipLaunchKernelGGL(calibration_slab_read_kernel, dim3((uint32_t)compute_units * blocks_per_cu), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const unsigned char*>(pool.ptr), static_cast<const uint32_t*>(slab_ids.ptr), num_slabs,
-                       static_cast<uint32_t*>(sink.ptr));
-    const hipError_t launched = hipGetLastError();
-    if (launched != hipSuccess) return fail(KHM_ERR_HIP, "calibration slab read launch failed: %s", hipGetErrorString(launched));
-    return KHM_OK;
+                       static_cast<const unsigned char*>(pool), slab_ids, num_slabs, sink);
+    return hipGetLastError() == hipSuccess ? 0 : 2;
 }

@@ -630,15 +630,6 @@ int khm_bidi_block_metadata_compute(const uint32_t* req_slots, uint32_t num_requ
                                     uint32_t* visible_kv_token_ranges, uint32_t* q_token_ranges, uint32_t* sdpa_map_task_templates,
                                     uint32_t* cu_sdpa_partial_outputs, khm_gqa_replay_shape* out_shape);
 
-/* ---- measurement aid (no counterpart in the reference) -------------------------------------------------------------------
- * Reads `num_slabs` slabs of 4096 bytes (16 token rows of one KV head at head_dim 128, bf16) of `pool`, slab i at byte
- * offset slab_ids[i] * 4096, with the lane layout and loads in flight of the split-KV Map kernel, from a resident grid of
- * `blocks_per_cu` blocks of 256 threads per compute unit, every wave the same share.  No arithmetic, no metadata chain, no
- * merge: its time for N bytes is what the memory system gives a launch of that size and access pattern, which the
- * benchmark reports beside the Map kernel's time for the same bytes.  `sink` (4 bytes) only keeps the loads alive. */
-int khm_calibration_slab_read(khm_buffer pool, khm_buffer slab_ids, uint32_t num_slabs, uint32_t blocks_per_cu, khm_buffer sink,
-                              void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -243,7 +243,6 @@ EXPORTED_SYMBOLS = (
     "khm_bidi_block_sdpa",
     "khm_bidi_block_capacity_new", "khm_bidi_block_select", "khm_bidi_block_metadata_compute",
     "khm_rms_norm_rope_yarn_correction_range", "khm_rms_norm_rope_kernel_parameters", "khm_rms_norm_rope",
-    "khm_calibration_slab_read",
     "khm_replay_bucket_policy_create", "khm_replay_bucket_policy_destroy", "khm_replay_bucket_policy_max_capacity",
     "khm_replay_bucket_policy_buckets", "khm_replay_bucket_policy_capacity", "khm_replay_bucket_policy_capacity_allow_zero",
     "khm_request_shapes_from_batch",
@@ -335,7 +334,6 @@ def lib() -> ctypes.CDLL:
     handle.khm_rms_norm_rope_kernel_parameters.argtypes = [ctypes.POINTER(RmsNormRopeConfig), float_p, u32, float_p]
     handle.khm_rms_norm_rope.argtypes = [ctypes.POINTER(RmsNormRopeConfig), u32, ctypes.POINTER(RmsNormRopeBuffers), ReplayU32,
                                          ctypes.c_void_p, ctypes.c_void_p]
-    handle.khm_calibration_slab_read.argtypes = [Buffer, Buffer, u32, u32, Buffer, ctypes.c_void_p]
     _lib = handle
     return handle
 

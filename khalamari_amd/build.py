@@ -26,7 +26,6 @@ SOURCES = [
     "kv_page_write.hip",
     "bidi_block_sdpa.hip",
     "rms_norm_rope.hip",
-    "calibration.hip",
 ]
 
 HIPCC_FLAGS = [
@@ -40,6 +39,21 @@ HIPCC_FLAGS = [
     # packed-FP32 VALU forms are kept off for every device function in this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+
+
+def build_bench_aid(verbose: bool = False) -> str:
+    """The read-only slab kernel bench.py times beside the Map kernels: a library of its own at the repository root,
+    not part of `libkhm_gqa_sdpa.so`."""
+    root = os.path.dirname(PACKAGE_DIR)
+    source, output = os.path.join(root, "bench_slab_read.hip"), os.path.join(root, "libbench_slab_read.so")
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    command = [hipcc, *HIPCC_FLAGS, "-x", "hip", source, "-o", output]
+    if verbose:
+        print(" ".join(command), flush=True)
+    result = subprocess.run(command, capture_output=True, text=True)
+    if result.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({result.returncode}):\n{result.stderr}")
+    return output
 
 
 def build(verbose: bool = False, extra_flags=(), output: str = LIB_PATH) -> str:
@@ -61,3 +75,4 @@ def build(verbose: bool = False, extra_flags=(), output: str = LIB_PATH) -> str:
 
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_bench_aid(verbose=True))

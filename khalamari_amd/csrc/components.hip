@@ -15,6 +15,7 @@ namespace khm {
 
 constexpr int kMapWaves = 4;
 
+
 typedef void (*MapKernel)(const MapParams);
 typedef void (*ReduceKernel)(const ReduceParams);
 

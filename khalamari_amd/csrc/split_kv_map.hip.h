@@ -578,8 +578,11 @@ __global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapPara
 
     // ---- fused Reduce: the last block of a (Q range, head group) merges all of its partial states ----------
     if (!fused) return;
-    // The partial state above went out through device-coherent stores.  The barrier's release makes every
-    // wave wait for its stores to complete before thread 0 signals arrival; no L2 write-back is involved.
+    // The partial state above went out through device-coherent stores.  Every thread releases its own stores at agent
+    // scope (a wait for them to complete: they bypass this XCD's L2, so nothing is written back), the barrier then
+    // orders all of them before thread 0 signals arrival, and the block that sees the last arrival acquires before it
+    // reads what the others stored.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     __syncthreads();
     uint32_t* flag_lds = reinterpret_cast<uint32_t*>(stats_lds);
     const uint32_t partial_begin = p.cu_partial_outputs[range_index];
@@ -587,13 +590,14 @@ __global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapPara
     if (partial_end > num_active_splits) partial_end = num_active_splits;
     if (tid == 0) {
         uint32_t* counter = p.arrival_counters + (uint64_t)range_index * gridDim.y + head_group_index;
-        const uint32_t arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+        const uint32_t arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) + 1u;
         const uint32_t last = arrived == partial_end - partial_begin ? 1u : 0u;
         if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // re-arm for the next launch
         flag_lds[0] = last;
     }
     __syncthreads();
     if (flag_lds[0] == 0u) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     {
         // Work units are (column, partial-slice) pairs; a group of D/4 lanes owns one unit at a time and walks
         // its partials with an online merge, eight partials' loads in flight at once.  With at least as many

@@ -227,8 +227,10 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     // Rounding a softmax weight to bf16 costs up to 2^-9 of that weight; with few keys the weights are O(1) and
     // the error shows at the 1e-3 level.  Blocks with a column that sees at most kPreciseSpan keys therefore feed the
     // second MFMA with hi + lo bf16 pairs (the reference keeps P in f32); long contexts, where every weight is small,
-    // use one.
-    constexpr uint32_t kPreciseSpan = 256;
+    // use one.  On N(0,1) data a column over n keys has about n / e keys of comparable weight, so single rounding leaves
+    // about 2^-9 / sqrt(3 n / e) of |v| in the output: 6e-4 at the worst of 4 million outputs with n just above 256
+    // (1.05 % of an output of 0.05), half that from 1024 keys on.
+    constexpr uint32_t kPreciseSpan = 1024;
     const bool precise = (uint32_t)__builtin_amdgcn_readfirstlane(min_span) <= kPreciseSpan;
     __syncthreads();   // range_lds is about to be overwritten by the first tile
     {

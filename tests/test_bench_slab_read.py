@@ -1,0 +1,25 @@
+"""bench.py's read-only slab launch (a library of its own beside bench.py): one run on the GPU."""
+import numpy as np
+import pytest
+
+import bench
+
+
+@pytest.mark.gpu
+def test_gpu_reads_listed_slabs_and_leaves_the_sink_alone(device):
+    import torch
+
+    slabs = 1024
+    pool = torch.randint(-2**31, 2**31 - 1, (slabs * bench.SLAB_BYTES // 4,), dtype=torch.int32, device=device)
+    order = np.random.default_rng(5).permutation(slabs).astype(np.uint32)
+    ids = torch.from_numpy(order.view(np.int32)).to(device)
+    sink = torch.zeros(1, dtype=torch.int32, device=device)
+    for count in (1, 3, slabs):   # fewer slabs than waves, and a full list
+        print(f"bench slab read: {count} slabs", flush=True)
+        bench.slab_read(pool, ids, count, sink, blocks_per_cu=2)
+    torch.cuda.synchronize()
+    assert int(sink.item()) == 0
+    with pytest.raises(RuntimeError):
+        bench.slab_read(pool, ids, 0, sink)          # nothing to read
+    with pytest.raises(RuntimeError):
+        bench.slab_read(pool, ids, 4, sink, blocks_per_cu=9)

@@ -1,8 +1,8 @@
 """Parity at the full sizes of the five benchmark configs.  The synthetic configs are built exactly as bench.py builds them (same seeds,
 page permutations and selector decisions), one step runs through the C ABI, and the output rows of sampled Q tokens are
-checked against the CPU oracle at the full context - every token where that takes seconds (configs 2 and 3), the
-first / middle / last token of each request otherwise (as the reference's bench gate samples them:
-benches/gqa/matrix.rs:116-151).  Two size-independent properties close the gap for the rows the oracle does not visit:
+checked against the CPU oracle at the full context - every token of configs 1 to 4, and 64 tokens of each request of
+config 5, chosen so that every offset 0..31 inside a 32-token Q tile and 64 different tiles per request are hit (the
+reference's bench gate samples first / middle / last: benches/gqa/matrix.rs:116-151).  Two size-independent properties close the gap for the rows the oracle does not visit:
 the result does not depend on how the KV range is partitioned, and rows of unsampled tokens are finite and non-trivial."""
 import numpy as np
 import pytest
@@ -36,10 +36,16 @@ def _oracle_rows(workload, pool, tokens):
 
 
 def _sampled_tokens(workload, per_request):
+    """Flat Q token indices: every token of a request with at most `per_request` tokens (or per_request == 0), otherwise
+    `per_request` of them: sample i sits at offset i % 32 of Q tile (i * 31) % tiles, plus the request's first and last."""
     starts = np.concatenate([[0], np.cumsum(workload.q_lens)])
     tokens = []
     for request, count in enumerate(workload.q_lens):
-        picks = sorted({0, count // 2, count - 1}) if per_request == 3 else range(count)
+        if per_request == 0 or count <= per_request:
+            picks = range(count)
+        else:
+            tiles = count // 32
+            picks = sorted({0, count - 1} | {((i * 31) % tiles) * 32 + i % 32 for i in range(per_request)})
         tokens.extend(int(starts[request] + i) for i in picks)
     return tokens
 
@@ -64,7 +70,9 @@ def test_decode_configs_at_full_size(device, index, fp8):
         # config 3: the gate sees the bf16-rounded attention output (gqa_activation_gate.metal:19-39)
         gate_bits = workload.gates.cpu().view(torch.int16).numpy().view(np.uint16)[tokens]
         expected = oracle.bf16_bits_to_f32(oracle.gate_bf16(oracle.f32_to_bf16_bits(expected), gate_bits))
-    print(helpers.assert_parity(actual[tokens], expected, f"config {index} full size"))
+    stats = helpers.assert_parity(actual[tokens], expected, f"config {index} full size")
+    print(stats)
+    helpers.record_parity(f"config{index}{'_fp8_pages' if fp8 else ''} full size, bf16 output, {len(tokens)} tokens", stats)
 
 
 @pytest.mark.parametrize("index,fp8", [(4, False), (4, True), (5, False), (5, True)])
@@ -73,10 +81,12 @@ def test_verify_and_prefill_configs_at_full_size(device, index, fp8):
     actual = _run_step(workload)
     assert np.isfinite(actual).all()
     assert (np.abs(actual).reshape(actual.shape[0], -1).max(axis=1) > 0).all()      # every token row was written
-    tokens = _sampled_tokens(workload, per_request=3)
+    tokens = _sampled_tokens(workload, per_request=64)
     print(f"config {index} fp8={fp8}: oracle over {len(tokens)} sampled tokens", flush=True)
     expected = _oracle_rows(workload, workload.kv_pools[0], tokens)
-    print(helpers.assert_parity(actual[tokens], expected, f"config {index} full size"))
+    stats = helpers.assert_parity(actual[tokens], expected, f"config {index} full size")
+    print(stats)
+    helpers.record_parity(f"config{index}{'_fp8_pages' if fp8 else ''} full size, bf16 output, {len(tokens)} tokens", stats)
 
 
 def test_partitioning_does_not_change_the_result_at_full_size(device):

@@ -267,6 +267,33 @@ def test_fused_gate_and_standalone_gate(device):
         assert np.all(got[active:] == 7.0)
 
 
+def test_device_gate_matches_the_oracle_on_every_bf16_gate_value(device):
+    """All 65 536 bf16 gate bit patterns, each against several attention values, bit for bit: the device evaluates the
+    exponential with v_exp_f32, the oracle with libm, and every intermediate is rounded to bf16
+    (gqa_activation_gate.metal:19-39), so the two can only differ where the two exponentials straddle a bf16 rounding
+    boundary - and nowhere do they.  NaN gates must give NaN (payloads are not compared)."""
+    gate_bits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    rng = np.random.default_rng(52)
+    attention_values = [np.full(65536, 0x3F80, dtype=np.uint16),                                   # 1.0: the sigmoid itself
+                        np.full(65536, 0xC2F7, dtype=np.uint16),                                   # -123.5
+                        oracle.f32_to_bf16_bits(rng.standard_normal(65536, dtype=np.float32)),
+                        oracle.f32_to_bf16_bits(rng.standard_normal(65536, dtype=np.float32) * 1e-3)]
+    gates = gpu_runner.to_device(gate_bits, device)
+    for attention_bits in attention_values:
+        attn = gpu_runner.to_device(attention_bits, device)
+        out = torch.zeros_like(attn)
+        activation_gate.invoke(DTYPE_BF16, 1, 256, 256, attn, gates, out, ReplayU32.fixed(256))
+        torch.cuda.synchronize()
+        got = out.cpu().numpy().view(np.uint16)
+        want = oracle.gate_bf16(attention_bits, gate_bits)
+        got_nan = (got & 0x7FFF) > 0x7F80
+        want_nan = (want & 0x7FFF) > 0x7F80
+        assert np.array_equal(got_nan, want_nan)
+        different = np.flatnonzero((got != want) & ~want_nan)
+        assert different.size == 0, (f"{different.size} gate patterns differ, first: gate=0x{gate_bits[different[0]]:04x} "
+                                     f"attention=0x{attention_bits[different[0]]:04x} got=0x{got[different[0]]:04x} want=0x{want[different[0]]:04x}")
+
+
 def test_selector_and_metadata_drive_the_kernels_end_to_end(device):
     """prepare (Selector::select -> GQAMetadataBuffers::update) then record (Map/Reduce or direct), as
     GQA::prepare / record_sdpa do (attn/gqa/backend.rs:255-286,438-542)."""
