@@ -234,6 +234,30 @@ int khm_sliced_kv_map_reduce(const khm_sliced_kv* compute, const khm_sliced_kv_m
                              khm_replay_u32 num_active_tokens, khm_replay_u32 num_active_kv_splits,
                              const uint32_t* replay_parameters, void* stream);
 
+/* khm_sliced_kv_map_reduce for callers that cannot allocate or pass a workspace: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its executor owns a Scratch,
+ * sliced_kv.rs:265-320).  The partial states and the arrival counters live in a device array owned by the library,
+ * khm_sliced_kv_static_scratch_bytes() = 16 MiB per GPU, held until the process ends; the call allocates and frees
+ * nothing and enqueues two kernels on `stream` (a clear of the arrival counters, then the fused Map + Reduce).
+ * A shape whose partial states (two f32 [M][Hq] statistics + partial_dtype [M][Hq][D], each rounded up to 256 bytes)
+ * exceed 16 MiB - 256 KiB, or whose arrival counters (u32 [T][Hkv * q_head_ranges]) exceed 256 KiB, is rejected with
+ * KHM_ERR_INVALID_ARGUMENT.  Every call on one GPU shares that GPU's array: calls that overlap in time on one GPU
+ * race, whatever their streams; calls on one stream, or otherwise ordered, are fine.  Results are those of
+ * khm_sliced_kv_map_reduce bit for bit. */
+typedef struct khm_sliced_kv_static_buffers {
+    khm_buffer q;                       /* io dtype [T][Hq][D] */
+    khm_buffer kv_pages;
+    khm_buffer req_slots;               /* u32 [T] */
+    khm_buffer page_ids;
+    khm_buffer sdpa_map_task_templates; /* u32 [M][3] */
+    khm_buffer cu_sdpa_partial_outputs; /* u32 [T+1] */
+    khm_buffer output;                  /* io dtype [T][Hq][D] */
+} khm_sliced_kv_static_buffers;
+uint64_t khm_sliced_kv_static_scratch_bytes(void);
+int khm_sliced_kv_map_reduce_static(const khm_sliced_kv* compute, const khm_sliced_kv_static_buffers* buffers,
+                                    khm_buffer gates, khm_replay_u32 page_table_index, khm_replay_u32 num_active_tokens,
+                                    khm_replay_u32 num_active_kv_splits, const uint32_t* replay_parameters, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Sliced-Q component: sdpa/sliced_q.rs (verify blocks and chunked prefill)
  * ------------------------------------------------------------------------------------------ */

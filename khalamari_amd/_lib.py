@@ -108,6 +108,11 @@ class SlicedKvReduceBuffers(ctypes.Structure):
         "partial_exp_sums", "partial_max_logits", "partial_output", "cu_sdpa_partial_outputs", "output")]
 
 
+class SlicedKvStaticBuffers(ctypes.Structure):
+    _fields_ = [(name, Buffer) for name in (
+        "q", "kv_pages", "req_slots", "page_ids", "sdpa_map_task_templates", "cu_sdpa_partial_outputs", "output")]
+
+
 class SlicedQMapBuffers(ctypes.Structure):
     _fields_ = [(name, Buffer) for name in (
         "q", "kv_pages", "req_slots", "page_ids", "visible_kv_token_ranges", "q_token_ranges", "sdpa_map_task_templates",
@@ -233,6 +238,7 @@ EXPORTED_SYMBOLS = (
     "khm_sliced_kv_partial_output_stats_bytes", "khm_sliced_kv_partial_output_bytes", "khm_sliced_kv_create",
     "khm_sliced_kv_destroy", "khm_sliced_kv_map_kernel_id", "khm_sliced_kv_reduce_kernel_id", "khm_sliced_kv_map",
     "khm_sliced_kv_reduce", "khm_sliced_kv_reduce_gated", "khm_sliced_kv_arrival_counters_bytes", "khm_sliced_kv_map_reduce",
+    "khm_sliced_kv_static_scratch_bytes", "khm_sliced_kv_map_reduce_static",
     "khm_sliced_q_partial_output_bytes", "khm_sliced_q_partial_output_stats_bytes", "khm_sliced_q_create",
     "khm_sliced_q_destroy", "khm_sliced_q_map_kernel_id", "khm_sliced_q_map", "khm_sliced_q_direct", "khm_sliced_q_reduce",
     "khm_sliced_q_arrival_counters_bytes", "khm_sliced_q_map_reduce",
@@ -305,6 +311,10 @@ def lib() -> ctypes.CDLL:
     handle.khm_sliced_kv_map_reduce.argtypes = [ctypes.c_void_p, ctypes.POINTER(SlicedKvMapBuffers),
                                                 ctypes.POINTER(SlicedKvReduceBuffers), Buffer, Buffer, ReplayU32, ReplayU32, ReplayU32,
                                                 ctypes.c_void_p, ctypes.c_void_p]
+    handle.khm_sliced_kv_static_scratch_bytes.restype = ctypes.c_uint64
+    handle.khm_sliced_kv_static_scratch_bytes.argtypes = []
+    handle.khm_sliced_kv_map_reduce_static.argtypes = [ctypes.c_void_p, ctypes.POINTER(SlicedKvStaticBuffers), Buffer, ReplayU32,
+                                                       ReplayU32, ReplayU32, ctypes.c_void_p, ctypes.c_void_p]
     handle.khm_sliced_q_map_reduce.argtypes = [ctypes.c_void_p, ctypes.POINTER(SlicedQMapBuffers),
                                                ctypes.POINTER(SlicedQReduceBuffers), Buffer, ReplayU32, ReplayU32, ReplayU32, ReplayU32,
                                                ctypes.c_void_p, ctypes.c_void_p]

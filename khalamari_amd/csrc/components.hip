@@ -420,6 +420,86 @@ extern "C" int khm_sliced_kv_map_reduce(const khm_sliced_kv* compute, const khm_
                                 stream, &fused);
 }
 
+// ---- the fused Map + Reduce without any caller-provided or allocated workspace ----------------------------------------
+// For callers that cannot allocate (HIP graph capture, tight serving loops): the partial states and the arrival
+// counters of khm_sliced_kv_map_reduce live in a file-scope device array instead of caller buffers.  Each GPU holds its own
+// copy of the array at its own address; the address is looked up once per device and only that pointer is ever handed
+// to kernels (the array's name is a host-side stand-in, not a device address).
+constexpr uint64_t kStaticScratchBytes = 16ull << 20;
+constexpr uint64_t kStaticCounterBytes = 256ull << 10;   // arrival counters: a fixed region at the start, never used for anything else
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static unsigned char* static_scratch_of_device[kMaxDevices];   // filled on a device's first call; one stream user per handle, as everywhere here
+
+__global__ __launch_bounds__(256) void clear_u32_kernel(uint32_t* words, uint32_t count) {
+    const uint32_t index = blockIdx.x * 256 + threadIdx.x;
+    if (index < count) words[index] = 0u;
+}
+
+static int static_scratch_pointer(unsigned char** out) {
+    int device = -1;
+    hipError_t status = hipGetDevice(&device);
+    if (status != hipSuccess) return fail(KHM_ERR_HIP, "hipGetDevice failed: %s", hipGetErrorString(status));
+    KHM_REQUIRE(device >= 0 && device < kMaxDevices, "device index %d is outside the static scratch table", device);
+    if (static_scratch_of_device[device] == nullptr) {
+        void* address = nullptr;
+        status = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
+        if (status != hipSuccess || address == nullptr)
+            return fail(KHM_ERR_HIP, "hipGetSymbolAddress(scratch) failed on device %d: %s", device, hipGetErrorString(status));
+        static_scratch_of_device[device] = static_cast<unsigned char*>(address);
+    }
+    *out = static_scratch_of_device[device];
+    return KHM_OK;
+}
+
+extern "C" uint64_t khm_sliced_kv_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int khm_sliced_kv_map_reduce_static(const khm_sliced_kv* compute, const khm_sliced_kv_static_buffers* buffers, khm_buffer gates,
+                                               khm_replay_u32 page_table_index, khm_replay_u32 num_active_tokens,
+                                               khm_replay_u32 num_active_kv_splits, const uint32_t* replay_parameters, void* stream) {
+    clear_error();
+    KHM_REQUIRE(compute != nullptr && buffers != nullptr, "compute and buffers must not be null");
+    const khm_gqa_sdpa_config& config = compute->config;
+    const khm_gqa_sdpa_shape& shape = compute->shape;
+    // the region layout: [arrival counters | exp sums | max logits | partial outputs], each 256-byte aligned
+    auto aligned = [](uint64_t bytes) { return (bytes + 255) & ~255ull; };
+    const uint64_t counter_bytes = khm_sliced_kv_arrival_counters_bytes(&config, &compute->variant, &shape);
+    const uint64_t stats_bytes = khm_sliced_kv_partial_output_stats_bytes(&config, &shape);
+    const uint64_t partial_bytes = khm_sliced_kv_partial_output_bytes(&config, &shape);
+    const uint64_t needed = kStaticCounterBytes + 2 * aligned(stats_bytes) + aligned(partial_bytes);
+    KHM_REQUIRE(counter_bytes <= kStaticCounterBytes && needed <= kStaticScratchBytes,
+                "shape needs %llu bytes of partial state and %llu bytes of arrival counters; the static scratch holds %llu and %llu: "
+                "use khm_sliced_kv_map_reduce with caller buffers",
+                (unsigned long long)(needed - kStaticCounterBytes), (unsigned long long)counter_bytes,
+                (unsigned long long)(kStaticScratchBytes - kStaticCounterBytes), (unsigned long long)kStaticCounterBytes);
+    unsigned char* base = nullptr;
+    if (int s = static_scratch_pointer(&base)) return s;
+    khm_sliced_kv_map_buffers map_buffers{};
+    map_buffers.q = buffers->q;
+    map_buffers.kv_pages = buffers->kv_pages;
+    map_buffers.req_slots = buffers->req_slots;
+    map_buffers.page_ids = buffers->page_ids;
+    map_buffers.sdpa_map_task_templates = buffers->sdpa_map_task_templates;
+    map_buffers.partial_exp_sums = khm_buffer{base + kStaticCounterBytes, stats_bytes};
+    map_buffers.partial_max_logits = khm_buffer{base + kStaticCounterBytes + aligned(stats_bytes), stats_bytes};
+    map_buffers.partial_output = khm_buffer{base + kStaticCounterBytes + 2 * aligned(stats_bytes), partial_bytes};
+    KHM_BUFFER_AT_LEAST(buffers->cu_sdpa_partial_outputs, ((uint64_t)shape.num_total_tokens + 1) * 4, "cu_sdpa_partial_outputs");
+    KHM_BUFFER_AT_LEAST(buffers->output, khm_gqa_sdpa_q_bytes(&config, &shape), "output");
+    if (gates.ptr != nullptr) KHM_BUFFER_AT_LEAST(gates, khm_gqa_sdpa_q_bytes(&config, &shape), "gates");
+    // The counters must start at zero.  A finished call leaves them zero, but the array is shared by every call on this
+    // GPU and an earlier call may have been abandoned half-way, so they are cleared here - by a kernel, not a memset
+    // node, so that the call can be captured into a HIP graph.
+    const uint32_t counters = (uint32_t)(counter_bytes / 4);
+    hipLaunchKernelGGL(clear_u32_kernel, dim3((counters + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       reinterpret_cast<uint32_t*>(base), counters);
+    if (int s = check_launch("static scratch clear")) return s;
+    const FusedReduceArgs fused{static_cast<const uint32_t*>(buffers->cu_sdpa_partial_outputs.ptr), reinterpret_cast<uint32_t*>(base),
+                                static_cast<uint16_t*>(buffers->output.ptr), static_cast<const uint16_t*>(gates.ptr)};
+    return launch_sliced_kv_map(compute, &map_buffers, page_table_index, num_active_tokens, num_active_kv_splits, replay_parameters,
+                                stream, &fused);
+}
+
 static int launch_sliced_kv_reduce(const khm_sliced_kv* compute, const khm_sliced_kv_reduce_buffers* buffers, const khm_buffer* gates,
                                    khm_replay_u32 num_active_tokens, const uint32_t* replay_parameters, void* stream) {
     KHM_REQUIRE(compute != nullptr && buffers != nullptr, "compute and buffers must not be null");

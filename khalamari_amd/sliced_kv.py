@@ -7,7 +7,7 @@ from dataclasses import dataclass, field
 from . import _lib
 from ._buffers import param_block, stream_handle, view
 from ._lib import (DTYPE_BF16, GqaSdpaConfig, GqaSdpaShape, PageTableLayout, ReplayU32, SdpaVariant,
-                   SlicedKvMapBuffers, SlicedKvReduceBuffers)
+                   SlicedKvMapBuffers, SlicedKvReduceBuffers, SlicedKvStaticBuffers)
 
 
 @dataclass(frozen=True)
@@ -147,6 +147,18 @@ class Compute:
                                                        gate_view, view(arrival_counters), page_table_index, num_active_tokens,
                                                        num_active_kv_splits, param_block(replay_parameters),
                                                        stream_handle(stream)))
+
+    def invoke_map_reduce_static(self, *, q, kv_pages, req_slots, page_ids, sdpa_map_task_templates, cu_sdpa_partial_outputs,
+                                 output, page_table_index: ReplayU32, num_active_tokens: ReplayU32,
+                                 num_active_kv_splits: ReplayU32, gates=None, replay_parameters=None, stream=None) -> None:
+        """`invoke_map_reduce` with the partial states and arrival counters in the library's own static device array:
+        nothing is allocated and no workspace is passed (no counterpart in the reference)."""
+        buffers = SlicedKvStaticBuffers(view(q), view(kv_pages), view(req_slots), view(page_ids), view(sdpa_map_task_templates),
+                                        view(cu_sdpa_partial_outputs), view(output))
+        gate_view = view(gates) if gates is not None else _lib.Buffer(None, 0)
+        _lib.check(_lib.lib().khm_sliced_kv_map_reduce_static(self._handle, ctypes.byref(buffers), gate_view, page_table_index,
+                                                              num_active_tokens, num_active_kv_splits,
+                                                              param_block(replay_parameters), stream_handle(stream)))
 
     def invoke_reduce(self, *, partial_exp_sums, partial_max_logits, partial_output, cu_sdpa_partial_outputs, output,
                       num_active_tokens: ReplayU32, gates=None, replay_parameters=None, stream=None) -> None:
