@@ -55,9 +55,10 @@ SLAB_BYTES = 4096
 _slab_reader_lib = None
 
 
-def slab_read(pool, slab_ids, num_slabs: int, sink, blocks_per_cu: int = 2) -> None:
-    """Enqueues, on torch's current stream, a launch that only reads `num_slabs` slabs of 4096 bytes of `pool` (slab i at
-    byte offset `slab_ids[i] * 4096`) from a resident grid, in the Map kernel's lane layout.  The kernel lives in
+def slab_read(pool, slab_ids, num_slabs: int, sink, blocks_per_cu: int = 2, run_slabs: int = 1) -> None:
+    """Enqueues, on torch's current stream, a launch that only reads `num_slabs` slabs of 4096 bytes of `pool` from a
+    resident grid, in the Map kernel's lane layout: slab i at byte offset `slab_ids[i] * 4096`, or with `run_slabs` > 1
+    runs of that many consecutive slabs, run j at `slab_ids[j] * run_slabs * 4096`.  The kernel lives in
     `libbench_slab_read.so` beside this file (source `bench_slab_read.hip`): a measurement aid, not part of the library."""
     import ctypes
 
@@ -71,13 +72,13 @@ def slab_read(pool, slab_ids, num_slabs: int, sink, blocks_per_cu: int = 2) -> N
         _slab_reader_lib = ctypes.CDLL(path)
         _slab_reader_lib.bench_slab_read.restype = ctypes.c_int
         _slab_reader_lib.bench_slab_read.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint32,
-                                                     ctypes.c_uint32, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
+                                                     ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
 
     def nbytes(t):
         return t.numel() * t.element_size()
 
     status = _slab_reader_lib.bench_slab_read(pool.data_ptr(), nbytes(pool), slab_ids.data_ptr(), nbytes(slab_ids), int(num_slabs),
-                                              int(blocks_per_cu), sink.data_ptr(), nbytes(sink),
+                                              int(run_slabs), int(blocks_per_cu), sink.data_ptr(), nbytes(sink),
                                               ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
     if status != 0:
         raise RuntimeError(f"bench_slab_read failed with status {status}")
@@ -512,6 +513,36 @@ def producer_rows(device, steps: int = 20) -> dict:
     return result
 
 
+def slab_run_table(device, index: int = 2, steps: int = 40) -> list:
+    """The read-only launch of a config's K/V bytes as contiguous runs of 4 .. 64 KB at random places of its pools: what a
+    block that covered several KV heads of a page (longer contiguous reads) could gain over 4 KB slabs."""
+    import torch
+
+    workload = Workload(index, device)
+    spec = workload.spec
+    kv_bytes = workload.visible_tokens * spec["hkv"] * spec["d"] * 2 * workload.kv_element_bytes
+    pool_slabs = workload.kv_pools[0].numel() * workload.kv_pools[0].element_size() // SLAB_BYTES
+    sink = torch.zeros(1, dtype=torch.int32, device=device)
+    rows = []
+    for run in (1, 2, 4, 8, 16):
+        num_slabs = (kv_bytes // SLAB_BYTES) // run * run
+        order = np.random.Generator(np.random.PCG64(1234)).permutation(pool_slabs // run)[:num_slabs // run].astype(np.uint32)
+        run_ids = torch.from_numpy(order.view(np.int32)).to(device)
+        for blocks_per_cu in (2, 4):
+            for i in range(3):
+                slab_read(workload.kv_pools[i % NUM_POOLS], run_ids, num_slabs, sink, blocks_per_cu, run)
+            pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+            for i, (a, b) in enumerate(pairs):
+                a.record()
+                slab_read(workload.kv_pools[i % NUM_POOLS], run_ids, num_slabs, sink, blocks_per_cu, run)
+                b.record()
+            torch.cuda.synchronize()
+            us = float(np.mean([a.elapsed_time(b) for a, b in pairs])) * 1e3
+            rows.append({"contiguous_kb": run * SLAB_BYTES // 1024, "blocks_per_cu": blocks_per_cu, "us": us,
+                         "gbps": num_slabs * SLAB_BYTES / us / 1e3})
+    return rows
+
+
 def _cpu_model() -> str:
     try:
         with open("/proc/cpuinfo") as handle:
@@ -549,6 +580,8 @@ def main() -> int:
                         help="time only the kernels that feed the SDPA (RMSNorm + RoPE, K/V page write) and print their JSON (profiling runs)")
     parser.add_argument("--fp8-pages", action="store_true",
                         help="headline config on FP8 E4M3FN pages, the reference's cache format (profiling runs; the default headline keeps bf16 pages)")
+    parser.add_argument("--slab-runs", action="store_true",
+                        help="time only the read-only launch of the headline config's K/V bytes as contiguous runs of 4 .. 64 KB and print the table as JSON")
     parser.add_argument("--calibration-copy", action="store_true",
                         help="also launch a plain 1 GiB copy kernel, the known-size reference for FETCH_SIZE / WRITE_SIZE counter runs")
     args = parser.parse_args()
@@ -566,6 +599,9 @@ def main() -> int:
         calibration_copy(device)
     if args.producers:
         print(json.dumps({"producers": producer_rows(device, steps=max(args.steps, 1))}))
+        return 0
+    if args.slab_runs:
+        print(json.dumps({"slab_runs": slab_run_table(device, args.config)}))
         return 0
     headline = Workload(args.config, device, fp8_pages=args.fp8_pages)
     head = headline.report(args.steps, args.warmup)

@@ -25,6 +25,42 @@ __device__ __forceinline__ uint32_t resolve_u32(DeviceReplayU32 r, const uint32_
     return r.is_parameter ? params[r.value] : r.value;
 }
 
+// A word of a table that does not change while the kernel runs, read with a wave-uniform index through the constant
+// address space: the compiler then issues a scalar load (its own counter) instead of a vector load, and consecutive ones
+// with no branch between them go out together and are waited for once.
+__device__ __forceinline__ uint32_t load_uniform_u32(const uint32_t* table, uint64_t index) {
+    typedef const uint32_t __attribute__((address_space(4))) * ConstantU32;
+    return ((ConstantU32)(uintptr_t)table)[index];
+}
+
+// Makes the kernel read its whole argument block when it starts.  Left alone, the compiler fetches each group of
+// arguments where it is first used, behind the branches of the task decode: two more dependent round trips to memory in
+// front of a block's first K/V load.
+__device__ __forceinline__ void fetch_all_arguments(const MapParams& p) {
+    asm volatile("" ::"s"(p.q), "s"(p.kv_pages), "s"(p.req_slots), "s"(p.page_ids), "s"(p.visible_ranges), "s"(p.q_token_ranges),
+                 "s"(p.templates), "s"(p.exp_sums), "s"(p.max_logits), "s"(p.out), "s"(p.replay_parameters));
+    asm volatile("" ::"s"(p.page_bytes), "s"(p.num_q_heads), "s"(p.num_kv_heads), "s"(p.q_heads_per_kv_head), "s"(p.max_q_heads),
+                 "s"(p.num_q_head_ranges), "s"(p.max_q_tokens), "s"(p.tokens_per_page), "s"(p.tokens_per_page_shift),
+                 "s"(p.num_gqa_layers), "s"(p.pages_per_request_layer), "s"(p.output_mode), "s"(p.scale_log2e));
+}
+
+// The four replay values of a Map launch, each fixed or read from the parameter block; the reads are issued together.
+struct ReplayValues {
+    uint32_t layer, num_active_tokens, num_active_q_token_tiles, num_active_kv_splits;
+};
+__device__ __forceinline__ ReplayValues resolve_replay_values(const MapParams& p) {
+    // with no parameter block every value is fixed and the words read here (any readable ones) are not used
+    const uint32_t* source = p.replay_parameters != nullptr ? p.replay_parameters : p.templates;
+    const uint32_t a = load_uniform_u32(source, p.layer_index.is_parameter ? p.layer_index.value : 0u);
+    const uint32_t b = load_uniform_u32(source, p.num_active_tokens.is_parameter ? p.num_active_tokens.value : 0u);
+    const uint32_t c = load_uniform_u32(source, p.num_active_q_token_tiles.is_parameter ? p.num_active_q_token_tiles.value : 0u);
+    const uint32_t d = load_uniform_u32(source, p.num_active_kv_splits.is_parameter ? p.num_active_kv_splits.value : 0u);
+    return ReplayValues{p.layer_index.is_parameter ? a : p.layer_index.value,
+                        p.num_active_tokens.is_parameter ? b : p.num_active_tokens.value,
+                        p.num_active_q_token_tiles.is_parameter ? c : p.num_active_q_token_tiles.value,
+                        p.num_active_kv_splits.is_parameter ? d : p.num_active_kv_splits.value};
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 // e^x through v_exp_f32; both Reduce implementations use this one so they agree bit for bit.
 __device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }

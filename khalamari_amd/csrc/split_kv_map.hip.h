@@ -100,26 +100,33 @@ __global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapPara
     const uint32_t linear_block = blockIdx.y * gridDim.x + blockIdx.x;
     const uint32_t task = linear_block / gridDim.y;
     const uint32_t head_group_index = linear_block % gridDim.y;
-    const uint32_t num_active_splits = resolve_u32(p.num_active_kv_splits, p.replay_parameters);
+    // The metadata chain in front of a block's first K/V load is a chain of dependent round trips to memory, a fifth of
+    // the life of a 512-token decode block: arguments -> task template -> request slot -> page ids -> K/V.  Every link is
+    // a scalar load, and everything that hangs on the same link is requested together: the whole argument block; then
+    // the template's three words and the replay values; then (sliced-Q) the Q range; then the request slot.  The grid
+    // has one block per template of the padded shape, so reading the template before the activity test is in bounds.
+    fetch_all_arguments(p);
+    const ReplayValues replay = resolve_replay_values(p);
+    const uint32_t range_index = load_uniform_u32(p.templates, 3 * (uint64_t)task);
+    const uint32_t kv_begin = load_uniform_u32(p.templates, 3 * (uint64_t)task + 1);
+    const uint32_t kv_end = load_uniform_u32(p.templates, 3 * (uint64_t)task + 2);
+    const uint32_t num_active_splits = replay.num_active_kv_splits;
     if (task >= num_active_splits) return;
-    const uint32_t range_index = p.templates[3 * (uint64_t)task];
-    if (range_index >= resolve_u32(p.num_active_q_token_tiles, p.replay_parameters)) return;
+    if (range_index >= replay.num_active_q_token_tiles) return;
     uint32_t flat_begin, flat_end;
     if (p.q_token_ranges != nullptr) {
-        flat_begin = p.q_token_ranges[2 * (uint64_t)range_index];
-        flat_end = p.q_token_ranges[2 * (uint64_t)range_index + 1];
+        flat_begin = load_uniform_u32(p.q_token_ranges, 2 * (uint64_t)range_index);
+        flat_end = load_uniform_u32(p.q_token_ranges, 2 * (uint64_t)range_index + 1);
     } else {
         flat_begin = range_index;
         flat_end = range_index + 1;
     }
-    const uint32_t num_active_tokens = resolve_u32(p.num_active_tokens, p.replay_parameters);
+    const uint32_t num_active_tokens = replay.num_active_tokens;
     if (flat_begin >= num_active_tokens || flat_end > num_active_tokens || flat_end <= flat_begin) return;
     uint32_t num_q = flat_end - flat_begin;
     if (num_q > p.max_q_tokens) num_q = p.max_q_tokens;
-    const uint32_t kv_begin = p.templates[3 * (uint64_t)task + 1];
-    const uint32_t kv_end = p.templates[3 * (uint64_t)task + 2];
-    const uint32_t req_slot = p.req_slots[flat_begin];
-    const uint32_t layer = resolve_u32(p.layer_index, p.replay_parameters);
+    const uint32_t req_slot = load_uniform_u32(p.req_slots, flat_begin);
+    const uint32_t layer = replay.layer;
 
     const uint32_t head_range = head_group_index % p.num_q_head_ranges;
     const uint32_t kv_head = head_group_index / p.num_q_head_ranges;
@@ -578,11 +585,14 @@ __global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapPara
 
     // ---- fused Reduce: the last block of a (Q range, head group) merges all of its partial states ----------
     if (!fused) return;
-    // The partial state above went out through device-coherent stores.  Every thread releases its own stores at agent
-    // scope (a wait for them to complete: they bypass this XCD's L2, so nothing is written back), the barrier then
-    // orders all of them before thread 0 signals arrival, and the block that sees the last arrival acquires before it
-    // reads what the others stored.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    // Publishing the partial state to whichever block merges it.  Every store above is a device-coherent (sc1,
+    // write-through) store: it is never held dirty in this XCD's L2, so what a release needs here is only that each wave
+    // waits until its own stores have been acknowledged - the explicit wait below, which does not depend on what the
+    // compiler puts in front of a barrier.  (A release fence at agent scope adds an L2 write-back per wave with nothing to
+    // write back, and that alone takes a 2272-block launch from 114 to 209 us.)  The barrier then orders all waves' stores
+    // before thread 0 signals arrival; the arrival is an acquire, so the block that sees the last one reads the others'
+    // partial states - through device-coherent loads - after their stores.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     uint32_t* flag_lds = reinterpret_cast<uint32_t*>(stats_lds);
     const uint32_t partial_begin = p.cu_partial_outputs[range_index];
@@ -590,14 +600,13 @@ __global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapPara
     if (partial_end > num_active_splits) partial_end = num_active_splits;
     if (tid == 0) {
         uint32_t* counter = p.arrival_counters + (uint64_t)range_index * gridDim.y + head_group_index;
-        const uint32_t arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+        const uint32_t arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) + 1u;
         const uint32_t last = arrived == partial_end - partial_begin ? 1u : 0u;
         if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // re-arm for the next launch
         flag_lds[0] = last;
     }
     __syncthreads();
     if (flag_lds[0] == 0u) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     {
         // Work units are (column, partial-slice) pairs; a group of D/4 lanes owns one unit at a time and walks
         // its partials with an online merge, eight partials' loads in flight at once.  With at least as many

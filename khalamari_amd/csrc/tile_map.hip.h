@@ -68,14 +68,6 @@ __device__ __forceinline__ void barrier_keeping_loads_in_flight() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-// A page-table entry read with a wave-uniform index.  The table does not change while the kernel runs, so it is
-// read through the constant address space: the compiler then issues a scalar load (its own counter) instead of a
-// vector load whose wait would also drain the K/V loads in flight.
-__device__ __forceinline__ uint32_t load_uniform_u32(const uint32_t* table, uint32_t index) {
-    typedef const uint32_t __attribute__((address_space(4))) * ConstantU32;
-    return ((ConstantU32)(uintptr_t)table)[index];
-}
-
 // KV8: the pages hold FP8 E4M3FN codes.  The LDS tiles stay bf16 in the same swizzled layout, so everything after the
 // load is unchanged; the tile itself travels through registers (16 bytes = 16 codes per lane and load), is decoded
 // there and written to LDS one barrier before it is first read.  One tile is in flight in registers while two are
@@ -130,19 +122,23 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     const uint32_t task = num_tasks - 1 - (uint32_t)(work % num_tasks);
 
     // ---- task decode (uniform) ---------------------------------------------------------------------------
-    if (task >= resolve_u32(p.num_active_kv_splits, p.replay_parameters)) return;
-    const uint32_t range_index = p.templates[3 * (uint64_t)task];
-    if (range_index >= resolve_u32(p.num_active_q_token_tiles, p.replay_parameters)) return;
-    const uint32_t flat_begin = p.q_token_ranges[2 * (uint64_t)range_index];
-    const uint32_t flat_end = p.q_token_ranges[2 * (uint64_t)range_index + 1];
-    const uint32_t num_active_tokens = resolve_u32(p.num_active_tokens, p.replay_parameters);
+    // every link of the chain arguments -> template -> Q range -> request slot is a scalar load, and what hangs on the
+    // same link is requested together (see split_kv_map_kernel)
+    fetch_all_arguments(p);
+    const ReplayValues replay = resolve_replay_values(p);
+    const uint32_t range_index = load_uniform_u32(p.templates, 3 * (uint64_t)task);
+    const uint32_t kv_begin = load_uniform_u32(p.templates, 3 * (uint64_t)task + 1);
+    const uint32_t kv_end = load_uniform_u32(p.templates, 3 * (uint64_t)task + 2);
+    if (task >= replay.num_active_kv_splits) return;
+    if (range_index >= replay.num_active_q_token_tiles) return;
+    const uint32_t flat_begin = load_uniform_u32(p.q_token_ranges, 2 * (uint64_t)range_index);
+    const uint32_t flat_end = load_uniform_u32(p.q_token_ranges, 2 * (uint64_t)range_index + 1);
+    const uint32_t num_active_tokens = replay.num_active_tokens;
     if (flat_begin >= num_active_tokens || flat_end > num_active_tokens || flat_end <= flat_begin) return;
     uint32_t num_q = flat_end - flat_begin;
     if (num_q > p.max_q_tokens) num_q = p.max_q_tokens;
-    const uint32_t kv_begin = p.templates[3 * (uint64_t)task + 1];
-    const uint32_t kv_end = p.templates[3 * (uint64_t)task + 2];
-    const uint32_t req_slot = p.req_slots[flat_begin];
-    const uint32_t layer = resolve_u32(p.layer_index, p.replay_parameters);
+    const uint32_t req_slot = load_uniform_u32(p.req_slots, flat_begin);
+    const uint32_t layer = replay.layer;
 
     const uint32_t head_range = head_group % p.num_q_head_ranges;
     const uint32_t kv_head = head_group / p.num_q_head_ranges;
