@@ -7,8 +7,14 @@
 // token's Q range (cu_sdpa_partial_outputs[range + 1] - 1), where the sliced-Q Reduce merges it with the history
 // partials.  Stored maxima are natural-log, like every partial of this ABI.
 //
-// One wavefront per (Q head, Q range, token offset), as in the reference (one SIMDgroup there): the work per task is
-// block_size x head_dim, far too little to tile; lanes stride over the head dimension.
+// Work shape on gfx950.  One 256-thread block per (Q range, KV head): the K and V rows of the request block under that KV
+// head are staged once in LDS as f32 (16-byte global loads, every Q head of the group and every token of the range reads
+// them from there), and the block's (token, Q head) tasks are served sixteen at a time, one task per 16-lane row of a
+// wave.  A lane keeps its eight-dim chunks of the Q row in registers (one 16-byte load per 128 dims), scores are dot
+// products over the lane's chunks summed across the row with DPP rotations, and the weighted V sum accumulates in
+// registers, eight dims per lane and chunk, stored with 16-byte stores.  Keys are walked in LDS-sized tiles with a
+// running maximum; a request block that fits one tile (the case the executor produces) is the reference's two passes:
+// maximum first, then weights, their sum and the weighted sum in key order.
 #include <hip/hip_runtime.h>
 
 #include "common.h"
@@ -38,68 +44,173 @@ struct BidiBlockParams {
     float scale;
 };
 
-template <typename T>
-__device__ __forceinline__ float load_value(const void* base, uint64_t index);
-template <>
-__device__ __forceinline__ float load_value<float>(const void* base, uint64_t index) {
-    return static_cast<const float*>(base)[index];
+// Sum over the sixteen lanes of a row, result in every lane of the row (DPP row rotations, no LDS).
+__device__ __forceinline__ float sum_within_row(float x) {
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x128, 0xf, 0xf, true));   // row_ror:8
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x124, 0xf, 0xf, true));   // row_ror:4
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x122, 0xf, 0xf, true));   // row_ror:2
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x121, 0xf, 0xf, true));   // row_ror:1
+    return x;
 }
-template <>
-__device__ __forceinline__ float load_value<uint16_t>(const void* base, uint64_t index) {
-    return bf16_bits_to_f32(static_cast<const uint16_t*>(base)[index]);
-}
-__device__ __forceinline__ void store_value(float* base, uint64_t index, float value) { base[index] = value; }
-__device__ __forceinline__ void store_value(uint16_t* base, uint64_t index, float value) { base[index] = f32_to_bf16_bits(value); }
 
-// T = float or uint16_t (bf16 bits).  Dynamic LDS: block_size floats (the logits, then the weights).
+// Eight consecutive values of a row as f32; T = float or uint16_t (bf16 bits).  `base` + `index` is 16-byte aligned.
 template <typename T>
-__global__ __launch_bounds__(64) void bidi_block_sdpa_kernel(const BidiBlockParams p) {
-    extern __shared__ float block_logits[];
-    const uint32_t lane = threadIdx.x;
-    const uint32_t q_head = blockIdx.x;
-    const uint32_t range = blockIdx.y;
+__device__ __forceinline__ void load_chunk(const void* base, uint64_t index, float (&out)[8]);
+template <>
+__device__ __forceinline__ void load_chunk<float>(const void* base, uint64_t index, float (&out)[8]) {
+    const f32x4 lo = *reinterpret_cast<const f32x4*>(static_cast<const float*>(base) + index);
+    const f32x4 hi = *reinterpret_cast<const f32x4*>(static_cast<const float*>(base) + index + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        out[i] = lo[i];
+        out[4 + i] = hi[i];
+    }
+}
+template <>
+__device__ __forceinline__ void load_chunk<uint16_t>(const void* base, uint64_t index, float (&out)[8]) {
+    const uint4 bits = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(base) + index);
+    const uint32_t words[4] = {bits.x, bits.y, bits.z, bits.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        out[2 * i] = bf16_bits_to_f32(words[i] & 0xffffu);
+        out[2 * i + 1] = bf16_bits_to_f32(words[i] >> 16);
+    }
+}
+__device__ __forceinline__ void store_chunk(float* base, uint64_t index, const float (&value)[8]) {
+    *reinterpret_cast<f32x4*>(base + index) = f32x4{value[0], value[1], value[2], value[3]};
+    *reinterpret_cast<f32x4*>(base + index + 4) = f32x4{value[4], value[5], value[6], value[7]};
+}
+__device__ __forceinline__ void store_chunk(uint16_t* base, uint64_t index, const float (&value)[8]) {
+    *reinterpret_cast<uint4*>(base + index) = make_uint4(pack_bf16x2(value[0], value[1]), pack_bf16x2(value[2], value[3]),
+                                                         pack_bf16x2(value[4], value[5]), pack_bf16x2(value[6], value[7]));
+}
+
+constexpr int kBidiThreads = 256;
+constexpr int kBidiTasksPerRound = kBidiThreads / 16;
+
+// T = float or uint16_t (bf16 bits); CHUNKS = ceil(head_dim / 128): eight-dim chunks per lane.  Dynamic LDS: K and V of
+// one key tile as f32, 2 * key_tile * head_dim floats.
+template <typename T, int CHUNKS>
+__global__ __launch_bounds__(kBidiThreads) void bidi_block_sdpa_kernel(const BidiBlockParams p, uint32_t key_tile) {
+    extern __shared__ __align__(16) float staged[];
+    const uint32_t range = blockIdx.x;
+    const uint32_t kv_head = blockIdx.y;
     if (range >= resolve_u32(p.num_active_q_token_ranges, p.replay_parameters)) return;
-    const uint32_t offset = blockIdx.z;
     const uint32_t flat_begin = p.q_token_ranges[2 * (uint64_t)range];
     const uint32_t flat_end = p.q_token_ranges[2 * (uint64_t)range + 1];
     // ranges and cumulative counts come from device memory: anything that points outside the buffers is skipped
-    if (flat_end <= flat_begin || flat_end > p.num_total_tokens || offset >= flat_end - flat_begin) return;
-    const uint32_t q_token = flat_begin + offset;
-    const uint32_t kv_head = q_head / (p.num_q_heads / p.num_kv_heads);
-    const uint32_t local_begin = (q_token / p.block_size) * p.block_size;
+    if (flat_end <= flat_begin || flat_end > p.num_total_tokens) return;
+    uint32_t num_q = flat_end - flat_begin;
+    if (num_q > p.max_q_tokens) num_q = p.max_q_tokens;
     const uint32_t slot = p.cu_partial_outputs[range + 1] - 1;
     if (slot >= p.num_total_partial_output_slots) return;
-    const uint64_t q_row = ((uint64_t)q_token * p.num_q_heads + q_head) * p.head_dim;
 
-    for (uint32_t local = 0; local < p.block_size; ++local) {
-        const uint64_t k_row = ((uint64_t)(local_begin + local) * p.num_kv_heads + kv_head) * p.head_dim;
-        float score = 0.0f;
-        for (uint32_t d = lane; d < p.head_dim; d += 64) score += load_value<T>(p.q, q_row + d) * load_value<T>(p.local_k, k_row + d);
+    const uint32_t D = p.head_dim, B = p.block_size;
+    const uint32_t group = p.num_q_heads / p.num_kv_heads;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t sub = tid & 15;                      // lane within the task's row
+    const uint32_t row_in_block = tid >> 4;             // which of the sixteen tasks of a round
+    float* k_lds = staged;                              // [key_tile][D]
+    float* v_lds = staged + (uint64_t)key_tile * D;
+    bool chunk_live[CHUNKS];
 #pragma unroll
-        for (int step = 32; step >= 1; step >>= 1) score += __shfl_xor(score, step);
-        if (lane == 0) block_logits[local] = score * p.scale;
-    }
-    __syncthreads();
-    float block_max = -INFINITY;
-    for (uint32_t local = 0; local < p.block_size; ++local) block_max = fmaxf(block_max, block_logits[local]);
-    __syncthreads();
-    // every lane derives the same weights; lane l rewrites entries l, l + 64, ...
-    float exp_sum = 0.0f;
-    for (uint32_t local = 0; local < p.block_size; ++local) exp_sum += __expf(block_logits[local] - block_max);
-    for (uint32_t local = lane; local < p.block_size; local += 64) block_logits[local] = __expf(block_logits[local] - block_max);
-    __syncthreads();
-    const uint64_t state = ((uint64_t)slot * p.num_q_heads + q_head) * p.max_q_tokens + offset;
-    if (lane == 0) {
-        p.exp_sums[state] = exp_sum;
-        p.max_logits[state] = block_max;
-    }
-    for (uint32_t d = lane; d < p.head_dim; d += 64) {
-        float output = 0.0f;
-        for (uint32_t local = 0; local < p.block_size; ++local) {
-            const uint64_t v_index = ((uint64_t)(local_begin + local) * p.num_kv_heads + kv_head) * p.head_dim + d;
-            output += block_logits[local] * load_value<T>(p.local_v, v_index);
+    for (int j = 0; j < CHUNKS; ++j) chunk_live[j] = (j * 16 + sub) * 8 < D;
+
+    // the tokens of a range lie in one request block when the executor built the ranges; any range is handled
+    const uint32_t first_block = flat_begin / B, last_block = (flat_begin + num_q - 1) / B;
+    for (uint32_t request_block = first_block; request_block <= last_block; ++request_block) {
+        const uint32_t local_begin = request_block * B;
+        const uint32_t token_lo = local_begin > flat_begin ? local_begin : flat_begin;
+        const uint32_t token_hi = local_begin + B < flat_begin + num_q ? local_begin + B : flat_begin + num_q;
+        const uint32_t num_tasks = (token_hi - token_lo) * group;
+        auto stage_tile = [&](uint32_t tile_begin, uint32_t tile_keys) __attribute__((always_inline)) {
+            __syncthreads();   // everyone is done with what the tile buffers held
+            for (uint32_t index = tid; index < tile_keys * (D / 8); index += kBidiThreads) {
+                const uint32_t key = index / (D / 8), chunk = index % (D / 8);
+                const uint64_t source = ((uint64_t)(local_begin + tile_begin + key) * p.num_kv_heads + kv_head) * D + chunk * 8;
+                float values[8];
+                load_chunk<T>(p.local_k, source, values);
+                store_chunk(k_lds, (uint64_t)key * D + chunk * 8, values);
+                load_chunk<T>(p.local_v, source, values);
+                store_chunk(v_lds, (uint64_t)key * D + chunk * 8, values);
+            }
+            __syncthreads();
+        };
+        // a request block that fits the tile buffers is staged once for all rounds of tasks
+        const bool single_tile = key_tile >= B;
+        if (single_tile) stage_tile(0, B);
+        for (uint32_t round = 0; round * kBidiTasksPerRound < num_tasks; ++round) {
+            const uint32_t task = round * kBidiTasksPerRound + row_in_block;
+            const bool live = task < num_tasks;
+            const uint32_t q_token = token_lo + (live ? task / group : 0u);
+            const uint32_t q_head = kv_head * group + (live ? task % group : 0u);
+            float q[CHUNKS][8], acc[CHUNKS][8];
+            const uint64_t q_row = ((uint64_t)q_token * p.num_q_heads + q_head) * D;
+#pragma unroll
+            for (int j = 0; j < CHUNKS; ++j) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) q[j][i] = acc[j][i] = 0.0f;
+                if (chunk_live[j]) load_chunk<T>(p.q, q_row + (j * 16 + sub) * 8, q[j]);
+            }
+            float run_max = -INFINITY, run_sum = 0.0f;
+            for (uint32_t tile_begin = 0; tile_begin < B; tile_begin += key_tile) {
+                const uint32_t tile_keys = B - tile_begin < key_tile ? B - tile_begin : key_tile;
+                if (!single_tile) stage_tile(tile_begin, tile_keys);
+                auto score_of = [&](uint32_t key) __attribute__((always_inline)) -> float {
+                    float part = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < CHUNKS; ++j) {
+                        if (chunk_live[j]) {
+                            float k_values[8];
+                            load_chunk<float>(k_lds, (uint64_t)key * D + (j * 16 + sub) * 8, k_values);
+#pragma unroll
+                            for (int i = 0; i < 8; ++i) part = __builtin_fmaf(q[j][i], k_values[i], part);
+                        }
+                    }
+                    return sum_within_row(part) * p.scale;
+                };
+                float tile_max = -INFINITY;
+                for (uint32_t key = 0; key < tile_keys; ++key) tile_max = fmaxf(tile_max, score_of(key));
+                const float next_max = fmaxf(run_max, tile_max);
+                const float keep = __expf(run_max - next_max);   // 0 before the first tile
+                run_sum *= keep;
+#pragma unroll
+                for (int j = 0; j < CHUNKS; ++j)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) acc[j][i] *= keep;
+                run_max = next_max;
+                for (uint32_t key = 0; key < tile_keys; ++key) {
+                    const float weight = __expf(score_of(key) - run_max);
+                    run_sum += weight;
+#pragma unroll
+                    for (int j = 0; j < CHUNKS; ++j) {
+                        if (chunk_live[j]) {
+                            float v_values[8];
+                            load_chunk<float>(v_lds, (uint64_t)key * D + (j * 16 + sub) * 8, v_values);
+#pragma unroll
+                            for (int i = 0; i < 8; ++i) acc[j][i] = __builtin_fmaf(weight, v_values[i], acc[j][i]);
+                        }
+                    }
+                }
+            }
+            if (live) {
+                const uint64_t state = ((uint64_t)slot * p.num_q_heads + q_head) * p.max_q_tokens + (q_token - flat_begin);
+                if (sub == 0) {
+                    p.exp_sums[state] = run_sum;
+                    p.max_logits[state] = run_max;
+                }
+                const float inverse = run_sum > 0.0f ? 1.0f / run_sum : 0.0f;
+#pragma unroll
+                for (int j = 0; j < CHUNKS; ++j) {
+                    if (chunk_live[j]) {
+                        float values[8];
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) values[i] = acc[j][i] * inverse;
+                        store_chunk(static_cast<T*>(p.partial_output), state * D + (j * 16 + sub) * 8, values);
+                    }
+                }
+            }
         }
-        store_value(static_cast<T*>(p.partial_output), state * p.head_dim + d, exp_sum > 0.0f ? output / exp_sum : 0.0f);
     }
 }
 
@@ -136,10 +247,8 @@ extern "C" int khm_bidi_block_sdpa(const khm_bidi_block_sdpa_config* config, con
                 "bidirectional block SDPA Q exceeds the shader u32 count domain");
     KHM_REQUIRE(product_fits_u32(shape->num_total_partial_output_slots, config->num_q_heads, config->max_q_tokens, config->head_dim),
                 "bidirectional block SDPA partial output exceeds the shader u32 element-index domain");
-    KHM_REQUIRE(config->max_q_tokens <= 65535 && shape->num_total_q_token_ranges <= 65535,
-                "bidirectional block SDPA grid exceeds 65535 in y or z");
-    KHM_REQUIRE((uint64_t)config->block_size * 4 <= 64 * 1024, "bidirectional block SDPA requires %u bytes of thread-block memory",
-                config->block_size * 4);
+    KHM_REQUIRE(config->num_kv_heads <= 65535, "bidirectional block SDPA grid exceeds 65535 KV heads");
+    if (config->head_dim > 1024) return fail(KHM_ERR_UNSUPPORTED, "no gfx950 bidirectional block SDPA kernel for head_dim %u (at most 1024)", config->head_dim);
     // Invocation::validate (bidi_block_sdpa.rs:289-333)
     if (!num_active_q_token_ranges.is_parameter) {
         KHM_REQUIRE(num_active_q_token_ranges.value == shape->num_total_q_token_ranges,
@@ -183,13 +292,21 @@ extern "C" int khm_bidi_block_sdpa(const khm_bidi_block_sdpa_config* config, con
     p.num_kv_heads = config->num_kv_heads;
     p.head_dim = config->head_dim;
     p.scale = config->scale;
-    const dim3 grid(config->num_q_heads, shape->num_total_q_token_ranges, config->max_q_tokens);
-    const uint32_t lds_bytes = config->block_size * 4;
-    if (config->dtype == KHM_DTYPE_F32) {
-        hipLaunchKernelGGL(bidi_block_sdpa_kernel<float>, grid, dim3(64), lds_bytes, static_cast<hipStream_t>(stream), p);
-    } else {
-        hipLaunchKernelGGL(bidi_block_sdpa_kernel<uint16_t>, grid, dim3(64), lds_bytes, static_cast<hipStream_t>(stream), p);
-    }
+    // key tile: as many keys as 48 KB of LDS hold as f32 K and V rows (a whole request block in every executor shape)
+    const uint32_t lds_budget = 48 * 1024;
+    uint32_t key_tile = lds_budget / (2 * config->head_dim * 4);
+    if (key_tile > config->block_size) key_tile = config->block_size;
+    const uint32_t lds_bytes = 2 * key_tile * config->head_dim * 4;
+    const dim3 grid(shape->num_total_q_token_ranges, config->num_kv_heads, 1);
+    const uint32_t chunks = (config->head_dim + 127) / 128;
+    typedef void (*Kernel)(const BidiBlockParams, uint32_t);
+    Kernel kernel = nullptr;
+    const bool f32 = config->dtype == KHM_DTYPE_F32;
+    if (chunks <= 1) kernel = f32 ? bidi_block_sdpa_kernel<float, 1> : bidi_block_sdpa_kernel<uint16_t, 1>;
+    else if (chunks <= 2) kernel = f32 ? bidi_block_sdpa_kernel<float, 2> : bidi_block_sdpa_kernel<uint16_t, 2>;
+    else if (chunks <= 4) kernel = f32 ? bidi_block_sdpa_kernel<float, 4> : bidi_block_sdpa_kernel<uint16_t, 4>;
+    else kernel = f32 ? bidi_block_sdpa_kernel<float, 8> : bidi_block_sdpa_kernel<uint16_t, 8>;
+    hipLaunchKernelGGL(kernel, grid, dim3(kBidiThreads), lds_bytes, static_cast<hipStream_t>(stream), p, key_tile);
     const hipError_t status = hipGetLastError();
     if (status != hipSuccess) return fail(KHM_ERR_HIP, "bidirectional block SDPA launch failed: %s", hipGetErrorString(status));
     return KHM_OK;

@@ -106,6 +106,61 @@ def test_gpu_matches_oracle_on_the_request_block_fixture(device, dtype_bf16):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("hq,hkv,d,block,max_q,dtype_bf16", [
+    (16, 2, 128, 8, 8, True),      # the executor's shape: eight tokens x eight heads = four rounds of sixteen tasks
+    (24, 4, 256, 16, 16, True),    # head_dim 256: two chunks per lane, 96 tasks per block
+    (24, 4, 256, 32, 8, False),    # f32, a 32-token request block of 256 dims: two key tiles (running maximum across tiles)
+    (6, 3, 96, 5, 4, True),        # head_dim that is not a multiple of 128, odd block size, ranges shorter than the block
+    (4, 1, 32, 40, 64, False),     # ranges that span request blocks (max_q_tokens above the block size)
+    (8, 2, 160, 12, 16, True),     # head_dim 160: the second chunk is live in four lanes of a row only
+])
+def test_gpu_matches_oracle_over_shapes(device, hq, hkv, d, block, max_q, dtype_bf16):
+    """Random request blocks through the C ABI against the oracle: several rounds of tasks per thread block, several key
+    tiles, partly filled lane rows, and Q ranges cut at max_q_tokens wherever they fall."""
+    import torch
+
+    from khalamari_amd import bidi_block_sdpa as bb
+
+    requests = 3
+    tokens = requests * block
+    rng = np.random.default_rng(hq * 1000 + d + block)
+    q = rng.standard_normal(tokens * hq * d).astype(np.float32)
+    k = rng.standard_normal(tokens * hkv * d).astype(np.float32)
+    v = rng.standard_normal(tokens * hkv * d).astype(np.float32)
+    if dtype_bf16:
+        q, k, v = oracle.bf16_round(q), oracle.bf16_round(k), oracle.bf16_round(v)
+    ranges = np.array([[begin, min(begin + max_q, tokens)] for begin in range(0, tokens, max_q)], dtype=np.uint32)
+    num_ranges = ranges.shape[0]
+    cu = np.arange(num_ranges + 1, dtype=np.uint32) * 2          # every range owns two slots; the block partial is the second
+    slots = 2 * num_ranges
+    scale = float(np.float32(d) ** np.float32(-0.5))
+    dtype = DTYPE_BF16 if dtype_bf16 else DTYPE_F32
+    config = bb.Config(block, max_q, hq, hkv, d, scale, dtype)
+    shape = bb.Shape(tokens, num_ranges, slots)
+    pack = (lambda a: oracle.f32_to_bf16_bits(a)) if dtype_bf16 else (lambda a: np.asarray(a, dtype=np.float32))
+    stats = config.partial_output_stat_elements(shape)
+    sums = torch.full((stats,), float("nan"), dtype=torch.float32, device=device)
+    maxs = torch.full((stats,), float("nan"), dtype=torch.float32, device=device)
+    partial = torch.zeros(config.partial_output_values(shape) * config.item_size(), dtype=torch.uint8, device=device)
+    print(f"bidi block shapes: hq={hq} hkv={hkv} d={d} block={block} max_q={max_q} bf16={dtype_bf16} ranges={num_ranges}", flush=True)
+    bb.Compute(config).invoke(shape, ReplayU32.fixed(num_ranges), q=_to(device, pack(q)), local_k=_to(device, pack(k)),
+                              local_v=_to(device, pack(v)), q_token_ranges=_to(device, ranges), cu_sdpa_partial_outputs=_to(device, cu),
+                              partial_exp_sums=sums, partial_max_logits=maxs, partial_output=partial)
+    torch.cuda.synchronize()
+    want_sums, want_maxs, want_out = oracle.bidi_block_sdpa(q, k, v, ranges, cu, num_ranges, block, max_q, hq, hkv, d, scale, slots)
+    got_sums = sums.cpu().numpy().reshape(want_sums.shape)
+    got_maxs = maxs.cpu().numpy().reshape(want_maxs.shape)
+    raw = partial.cpu().numpy()
+    got_out = (oracle.bf16_bits_to_f32(raw.view(np.uint16)) if dtype_bf16 else raw.view(np.float32)).reshape(want_out.shape)
+    written = ~np.isnan(want_sums)
+    assert written.sum() == tokens * hq
+    assert np.array_equal(np.isnan(got_sums), ~written)
+    assert np.abs(got_sums[written] - want_sums[written]).max() < 1e-4 * max(1.0, float(want_sums[written].max()))
+    assert np.abs(got_maxs[written] - want_maxs[written]).max() < 1e-4
+    assert np.abs(got_out[written] - want_out[written]).max() < (1e-2 if dtype_bf16 else 2e-5)
+
+
+@pytest.mark.gpu
 def test_gpu_replay_active_q_token_ranges(device):
     """test_replay_active_q_token_ranges_match_cpu_reference (bidi_block_sdpa_test.rs:50-157)."""
     import torch
