@@ -30,9 +30,9 @@
 
 namespace khm {
 
-template <int D, int BK, int NSTAGES>
+template <int D, int BK, int NSTAGES, int ROW_BYTES = D * 2>
 struct TileSmem {
-    static constexpr int kRowBytes = D * 2;
+    static constexpr int kRowBytes = ROW_BYTES;
     static constexpr int kTileBytes = BK * kRowBytes;
     static constexpr int kBytes = 2 /*K,V*/ * NSTAGES * kTileBytes;
 };
@@ -68,10 +68,16 @@ __device__ __forceinline__ void barrier_keeping_loads_in_flight() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-// KV8: the pages hold FP8 E4M3FN codes.  The LDS tiles stay bf16 in the same swizzled layout, so everything after the
-// load is unchanged; the tile itself travels through registers (16 bytes = 16 codes per lane and load), is decoded
-// there and written to LDS one barrier before it is first read.  One tile is in flight in registers while two are
-// consumed: enough for the MFMA-bound prefill tiles this mode is built for.
+// KV8: the pages hold FP8 E4M3FN codes, in one of two ways.
+// Tiles with two column tiles per wave (MFMA-bound prefill) keep their LDS tiles bf16 in the same swizzled layout, so
+// everything after the load is unchanged; the tile travels through registers (16 bytes = 16 codes per lane and load), is
+// decoded there once and written to LDS one barrier before it is first read.  One tile is in flight in registers while
+// two are consumed.
+// Tiles with one column tile per wave (bandwidth-bound verify blocks) keep the raw codes in LDS: the tile goes from
+// HBM/L2 straight into LDS like a bf16 one, half the bytes, and every wave decodes the fragments it reads (a K fragment
+// is one ds_read_b64, a V^T fragment one ds_read_b64_tr_b8, four conversions each).  That repeats the decode in each of
+// the four waves, which these tiles have the VALU time for, and takes the chain load -> registers -> decode -> LDS ->
+// barrier off the critical path of a tile.
 // DIRECT: the instantiation only ever writes final output (p.output_mode == kMapDirectBf16, which the host guarantees);
 // it exists where following the largest score is worth compiling out, see the untracked slices below.
 template <int D, int NTW, int NWAVES, int BK, int NSTAGES, int MIN_BLOCKS, bool KV8 = false, bool DIRECT = false>
@@ -87,9 +93,16 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     constexpr int LPW = 2 * UPW;                    // K + V loads per wave and tile
     static_assert(UNITS % NWAVES == 0 && UPW >= 1, "tile loads must divide evenly over the waves");
     static_assert((SL == 1 || SL == 2) && NSTAGES >= 3 && NSTAGES <= 5, "unsupported tiling");
-    static_assert(!KV8 || NSTAGES == 4, "the register-staged FP8 path is written for a ring of four tiles");
-    using Smem = TileSmem<D, BK, NSTAGES>;
+    constexpr bool RAW8 = KV8 && NTW == 1 && NWAVES == 4;   // raw FP8 codes in LDS, decoded by the waves that read them
+    constexpr bool STAGED8 = KV8 && !RAW8;       // FP8 tiles decoded once on their way into bf16 LDS tiles
+    static_assert(!STAGED8 || NSTAGES == 4, "the register-staged FP8 path is written for a ring of four tiles");
+    using Smem = TileSmem<D, BK, NSTAGES, RAW8 ? D : 2 * D>;
     constexpr int ROW = Smem::kRowBytes;
+    // XOR swizzle of the 16-byte chunk position inside an LDS row, by tile row.  bf16 rows (and raw rows of 256 bytes)
+    // alias bank for bank, so K reads spread sixteen rows over sixteen positions and the transposed V reads eight rows
+    // over every second one; raw rows of 128 bytes alias in pairs and have eight chunks: both planes use (row / 2) % 8.
+    auto k_swizzle_of = [](uint32_t row) -> uint32_t { return (RAW8 && D == 128) ? ((row >> 1) & 7u) : (row & 15u); };
+    auto v_swizzle_of = [](uint32_t row) -> uint32_t { return RAW8 ? (D == 128 ? ((row >> 1) & 7u) : (row & 15u)) : ((row & 7u) << 1); };
 
     extern __shared__ __align__(1024) unsigned char tile_smem[];
     unsigned char* k_lds = tile_smem;                                    // [NSTAGES][BK][ROW]
@@ -299,9 +312,9 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
 #pragma unroll
         for (int i = 0; i < UPW; ++i) {
             const uint32_t row = (wave * UPW + i) * RPL + load_row;                // row inside the tile
-            const uint32_t in_page = ((first_token + row) & (tpp - 1)) * ROW;
-            k_lane_offset[i] = in_page + ((load_pos ^ (row & 15)) << 4);
-            v_lane_offset[i] = in_page + ((load_pos ^ ((row & 7) << 1)) << 4);
+            const uint32_t in_page = ((first_token + row) & (tpp - 1)) * PAGE_ROW;
+            k_lane_offset[i] = in_page + ((load_pos ^ k_swizzle_of(row)) << 4);
+            v_lane_offset[i] = in_page + ((load_pos ^ v_swizzle_of(row)) << 4);
         }
     }
     auto issue_tile = [&](uint32_t tile, const TileIds ids) __attribute__((always_inline)) {
@@ -328,9 +341,9 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             token = token < blk_lo ? blk_lo : token;
             token = token >= blk_hi ? blk_hi - 1 : token;
             const unsigned char* page = p.kv_pages + (uint64_t)ids[i] * p.page_bytes;
-            const uint32_t in_page = (token & (tpp - 1)) * ROW;
-            const uint32_t k_offset_bytes = in_page + ((load_pos ^ (row & 15)) << 4);
-            const uint32_t v_offset_bytes = in_page + ((load_pos ^ ((row & 7) << 1)) << 4);
+            const uint32_t in_page = (token & (tpp - 1)) * PAGE_ROW;
+            const uint32_t k_offset_bytes = in_page + ((load_pos ^ k_swizzle_of(row)) << 4);
+            const uint32_t v_offset_bytes = in_page + ((load_pos ^ v_swizzle_of(row)) << 4);
             load_to_lds_b128(page + plane_k, k_offset_bytes, k_lds_address + stage * Smem::kTileBytes + unit * 1024);
             load_to_lds_b128(page + plane_v, v_offset_bytes, v_lds_address + stage * Smem::kTileBytes + unit * 1024);
         }
@@ -338,7 +351,7 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
 
     // FP8 pages: one tile in registers, decoded into the bf16 LDS layout the direct loads would have produced
     // (source chunk c of a K row lands at position c ^ (row & 15), of a V row at c ^ 2 (row & 7)).
-    uint4 raw_k[KV8 ? UPW : 1], raw_v[KV8 ? UPW : 1];
+    uint4 raw_k[STAGED8 ? UPW : 1], raw_v[STAGED8 ? UPW : 1];
     auto load_raw_tile = [&](uint32_t tile, const TileIds ids) __attribute__((always_inline)) {
         const uint32_t load_row = lane / CPR;
         const uint32_t load_pos = lane % CPR;
@@ -374,14 +387,36 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
 
     // ---- LDS read addresses (per lane, relative to the slice) -------------------------------------------------------
     // K: lane (r16, g) reads row rt*16 + r16, source chunk ks*4 + g, stored at position chunk ^ r16.
+    // Raw FP8 rows: the lane's eight codes of k-step ks are half of source chunk ks*2 + g/2, stored at that index XOR the
+    // row's swizzle (row tiles are sixteen rows apart, which leaves the swizzle alone).
     uint32_t k_offset[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) k_offset[ks] = r16 * ROW + (((ks * 4 + g) ^ r16) << 4);
+    for (int ks = 0; ks < KS; ++ks) {
+        if constexpr (RAW8) k_offset[ks] = r16 * ROW + ((((uint32_t)ks * 2 + (g >> 1)) ^ k_swizzle_of(r16)) << 4) + (g & 1) * 8;
+        else k_offset[ks] = r16 * ROW + (((ks * 4 + g) ^ r16) << 4);
+    }
     // V: lane (g, r) passes row 4g + r/4 (+16 for the second half), dims mt*16 + 4*(r%4) .. +3, i.e. source chunk
     // 2*mt + (r%4)/2, stored at position chunk ^ 2*(row & 7).
-    const uint32_t v_row = g * 4 + (r16 >> 2);
-    const uint32_t v_swizzle = ((r16 & 3) >> 1) ^ ((v_row & 7) << 1);
+    // Raw FP8 rows (ds_read_b64_tr_b8: lane r of a 16-lane group passes eight consecutive bytes; lane i receives byte i % 8
+    // of the rows passed by lanes i/8, i/8 + 2, ... i/8 + 14): lanes 2j and 2j + 1 pass the two halves of the sixteen
+    // dims of token (j < 4 ? 4g + j : 16 + 4g + j - 4), so lane r receives dim mt*16 + r of exactly the eight tokens whose
+    // weights it holds, in their order.
+    const uint32_t v_row = RAW8 ? ((r16 >> 1) < 4 ? g * 4 + (r16 >> 1) : 16 + g * 4 + (r16 >> 1) - 4) : g * 4 + (r16 >> 2);
+    const uint32_t v_swizzle = RAW8 ? v_swizzle_of(v_row) : ((r16 & 3) >> 1) ^ ((v_row & 7) << 1);
     const uint32_t v_base = v_row * ROW + (r16 & 1) * 8;
+    auto v_fragment = [&](const unsigned char* v_src, int mt) __attribute__((always_inline)) -> bf16x8 {
+        if constexpr (RAW8) {
+            typedef int CodeWords __attribute__((ext_vector_type(2)));
+            const unsigned char* address = v_src + v_base + (((uint32_t)mt ^ v_swizzle) << 4);
+            const CodeWords codes = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CodeWords __attribute__((address_space(3)))*)(address));
+            return __builtin_bit_cast(bf16x8, fp8x8_to_bf16x8(make_uint2((uint32_t)codes[0], (uint32_t)codes[1])));
+        } else {
+            const unsigned char* address = v_src + v_base + (((mt * 2) ^ v_swizzle) << 4);
+            const uint2 lo = __builtin_bit_cast(uint2, lds_read_tr16(address));
+            const uint2 hi = __builtin_bit_cast(uint2, lds_read_tr16(address + 16 * ROW));
+            return __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
+        }
+    };
 
     // ---- online-softmax state ------------------------------------------------------------------------------
     // Everything is kept in the log2 domain relative to ref[nt], the exponent reference of the lane's column.  The
@@ -421,8 +456,12 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
             for (int rt = 0; rt < 2; ++rt) {
-                const uint4 bits = *reinterpret_cast<const uint4*>(k_src + k_offset[ks] + rt * 16 * ROW);
-                const bf16x8 a = __builtin_bit_cast(bf16x8, bits);
+                bf16x8 a;
+                if constexpr (RAW8) {
+                    a = __builtin_bit_cast(bf16x8, fp8x8_to_bf16x8(*reinterpret_cast<const uint2*>(k_src + k_offset[ks] + rt * 16 * ROW)));
+                } else {
+                    a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(k_src + k_offset[ks] + rt * 16 * ROW));
+                }
 #pragma unroll
                 for (int nt = 0; nt < NTW; ++nt)
                     out.s[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, q_frag[nt][ks]), out.s[rt][nt], 0, 0, 0);
@@ -574,10 +613,7 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         // O^T += V^T . P^T over the 32 tokens: k = 8g + j <-> token (j < 4 ? 4g + j : 16 + 4g + j - 4) of the slice.
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            const unsigned char* address = v_src + v_base + (((mt * 2) ^ v_swizzle) << 4);
-            const uint2 lo = __builtin_bit_cast(uint2, lds_read_tr16(address));
-            const uint2 hi = __builtin_bit_cast(uint2, lds_read_tr16(address + 16 * ROW));
-            const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
+            const bf16x8 a = v_fragment(v_src, mt);
 #pragma unroll
             for (int nt = 0; nt < NTW; ++nt) {
                 const uint4 b_bits = make_uint4(p_bits[nt][0], p_bits[nt][1], p_bits[nt][2], p_bits[nt][3]);
@@ -625,7 +661,7 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     };
     auto run_tiles = [&](auto precise_tag, auto masked_tag, auto untracked_tag, uint32_t tile_begin, uint32_t tile_end) __attribute__((always_inline)) {
         for (uint32_t tile = tile_begin; tile < tile_end; ++tile) {
-            if constexpr (KV8) {
+            if constexpr (STAGED8) {
                 // tile + 1 was written to LDS during the previous tile; tile + 2 sits in registers, tile + 3 is requested
                 barrier_keeping_loads_in_flight();
                 if constexpr (!kRawTileBehindScores) advance_raw_tiles(tile);
@@ -644,13 +680,13 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             // this tile rather than straight after the barrier, where all waves would do address arithmetic at once
             // with the matrix pipe idle.
             auto request_next = [&]() __attribute__((always_inline)) {
-                if constexpr (!KV8) {
+                if constexpr (!STAGED8) {
                     if (tile + NSTAGES - 1 < num_tiles) {
                         issue_tile(tile + NSTAGES - 1, upcoming);
                         upcoming = fetch_ids(tile + NSTAGES);
                     }
                 }
-                if constexpr (KV8 && kRawTileBehindScores) advance_raw_tiles(tile);
+                if constexpr (STAGED8 && kRawTileBehindScores) advance_raw_tiles(tile);
             };
             auto nothing = []() __attribute__((always_inline)) {};
 #pragma unroll
@@ -665,7 +701,7 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         }
     };
     if (num_tiles > 0) {
-        if constexpr (KV8) {
+        if constexpr (STAGED8) {
             // tiles 0 and 1 into LDS, tile 2 into registers
             load_raw_tile(0, fetch_ids(0));
             write_raw_tile(0);
@@ -685,7 +721,7 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         if (wave_idle) {
             // the loads, waits and barriers of run_tiles, nothing else
             for (uint32_t tile = 0; tile < num_tiles; ++tile) {
-                if constexpr (KV8) {
+                if constexpr (STAGED8) {
                     barrier_keeping_loads_in_flight();
                     advance_raw_tiles(tile);
                 } else {
