@@ -52,6 +52,7 @@ CONFIGS[EXTRA_PREFILL_D256] = dict(name="extra: B=8 chunked prefill, 2048-token 
 
 
 SLAB_BYTES = 4096
+CLOCK_PROBE = True   # --no-clock-probe: counter runs want the Map launches alone on the device
 _slab_reader_lib = None
 
 
@@ -473,10 +474,11 @@ class Workload:
                           map_tflops=flops / (map_ms * 1e-3) / 1e12)
             result["roofline_frac"] = result["map_tflops"] / MFMA_BF16_PEAK_TFLOPS
             # the published peak is 256 CUs x 4 SIMDs x 1024 flop/clk at 2.4 GHz; the chip runs this kernel at a lower clock
-            clock_ghz = self.shader_clock_during_map(map_ms)
-            result["shader_clock_ghz"] = clock_ghz
-            result["mfma_peak_at_shader_clock_tflops"] = MFMA_BF16_PEAK_TFLOPS * clock_ghz / 2.4
-            result["frac_of_peak_at_shader_clock"] = result["map_tflops"] / result["mfma_peak_at_shader_clock_tflops"]
+            if CLOCK_PROBE:
+                clock_ghz = self.shader_clock_during_map(map_ms)
+                result["shader_clock_ghz"] = clock_ghz
+                result["mfma_peak_at_shader_clock_tflops"] = MFMA_BF16_PEAK_TFLOPS * clock_ghz / 2.4
+                result["frac_of_peak_at_shader_clock"] = result["map_tflops"] / result["mfma_peak_at_shader_clock_tflops"]
         else:
             nbytes = self.algorithmic_bytes()
             result.update(bound="hbm", algorithmic_bytes=nbytes, gbps=nbytes / (ms * 1e-3) / 1e9,
@@ -675,6 +677,8 @@ def main() -> int:
                         help="time only the read-only launch of the headline config's K/V bytes as contiguous runs of 4 .. 64 KB and print the table as JSON")
     parser.add_argument("--mfma-sustained", action="store_true",
                         help="time only the loop of bare bf16 MFMA instructions (rate and shader clock on constant and on random operands) and print the table as JSON")
+    parser.add_argument("--no-clock-probe", action="store_true",
+                        help="prefill configs: skip the one-wave shader clock probe that runs beside extra Map launches (profiling runs)")
     parser.add_argument("--calibration-copy", action="store_true",
                         help="also launch a plain 1 GiB copy kernel, the known-size reference for FETCH_SIZE / WRITE_SIZE counter runs")
     args = parser.parse_args()
@@ -688,6 +692,9 @@ def main() -> int:
         print("bench.py needs an MI355X (no GPU visible)", file=sys.stderr)
         return 2
     device = torch.device("cuda:0")
+    if args.no_clock_probe:
+        global CLOCK_PROBE
+        CLOCK_PROBE = False
     if args.calibration_copy:
         calibration_copy(device)
     if args.producers:

@@ -23,6 +23,16 @@ def test_library_exports_every_declared_symbol():
     assert b"gfx950" in lib.khm_version()
 
 
+def test_reference_side_binding_lists_every_declared_function():
+    """The Rust `extern "C"` block a maintainer would add names every function of the header."""
+    header = open(os.path.join(ROOT, "include", "khm_gqa_sdpa.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(khm_[a-z0-9_]+)\s*\(", header))
+    binding = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    bound = set(re.findall(r"pub fn (khm_[a-z0-9_]+)\(", binding))
+    assert declared == bound, f"only in the header: {sorted(declared - bound)}; only in the binding: {sorted(bound - declared)}"
+
+
 def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "_lib", None)
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libkhm_gqa_sdpa.so")
