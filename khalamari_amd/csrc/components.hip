@@ -19,27 +19,16 @@ constexpr int kMapWaves = 4;
 typedef void (*MapKernel)(const MapParams);
 typedef void (*ReduceKernel)(const ReduceParams);
 
+// Split-KV kernel (waves share nothing); K/V pages bf16 or FP8 E4M3FN.  Every variant that reaches it has one 16-column
+// tile: sliced-KV variants carry at most 8 Q heads and sliced-Q variants come here with at most 16 coordinates.
 template <bool KV8>
 static MapKernel small_tile_kernel_of(uint32_t head_dim, uint32_t column_tiles) {
-    if (head_dim == 128) {
-        switch (column_tiles) {
-            case 1: return split_kv_map_kernel<128, 1, kMapWaves, KV8>;
-            case 2: return split_kv_map_kernel<128, 2, kMapWaves, KV8>;
-            case 3: return split_kv_map_kernel<128, 3, kMapWaves, KV8>;
-            case 4: return split_kv_map_kernel<128, 4, kMapWaves, KV8>;
-        }
-    } else if (head_dim == 256) {
-        switch (column_tiles) {
-            case 1: return split_kv_map_kernel<256, 1, kMapWaves, KV8>;
-            case 2: return split_kv_map_kernel<256, 2, kMapWaves, KV8>;
-            case 3: return split_kv_map_kernel<256, 3, kMapWaves, KV8>;
-            case 4: return split_kv_map_kernel<256, 4, kMapWaves, KV8>;
-        }
-    }
+    if (column_tiles != 1) return nullptr;
+    if (head_dim == 128) return split_kv_map_kernel<128, 1, kMapWaves, KV8>;
+    if (head_dim == 256) return split_kv_map_kernel<256, 1, kMapWaves, KV8>;
     return nullptr;
 }
 
-// Split-KV kernel (waves share nothing) for up to 64 Q coordinates; K/V pages bf16 or FP8 E4M3FN.
 static MapKernel select_small_tile_kernel(uint32_t head_dim, uint32_t column_tiles, uint32_t kv_dtype) {
     return kv_dtype == KHM_DTYPE_FP8_E4M3FN ? small_tile_kernel_of<true>(head_dim, column_tiles)
                                             : small_tile_kernel_of<false>(head_dim, column_tiles);
