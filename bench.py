@@ -31,7 +31,7 @@ NUM_POOLS = 3
 # HBM bytes per Map launch from the hardware counters, (FETCH_SIZE * 2.000 + WRITE_SIZE * 1.000) KiB per dispatch:
 # two `rocprofv3 --pmc` runs per config, each counter scaled by what it reads for a plain 1 GiB copy kernel
 # (`--calibration-copy`).  The summaries with their commands are the text files under profiles/.
-MEASURED_MAP_TRAFFIC_BYTES = {2: 564_400_278, 3: 2_151_706_756, 4: 1_450_903_589, 5: 2_527_342_301}
+MEASURED_MAP_TRAFFIC_BYTES = {2: 564_421_875, 3: 2_151_671_477, 4: 1_451_466_787, 5: 1_201_877_171}
 
 CONFIGS = {
     1: dict(name="config1: B=1 q=1 Hq32/Hkv8/D128 ctx 1024, identity pages", hq=32, hkv=8, d=128, kind="decode", kv_slice=64),
@@ -430,7 +430,7 @@ class Workload:
     def shader_clock_during_map(self, map_ms: float) -> float:
         """GHz of the shader clock while the Map kernel runs: a one-wave kernel on a second stream (`bench_clock_probe`)
         compares the shader clock counter with the constant 100 MHz counter over a window that lies inside a row of
-        back-to-back Map launches."""
+        back-to-back Map launches.  It reads the XCD it lands on; runs differ by about 0.1 GHz."""
         import ctypes
 
         import torch

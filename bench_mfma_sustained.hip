@@ -69,8 +69,9 @@ __global__ __launch_bounds__(kThreads) void mfma_sustained_kernel(const uint4* o
 }
 
 // One wave that sleeps for `delay_ticks` of the 100 MHz counter, then reads both counters, sleeps for `window_ticks`
-// and reads them again: launched on a second stream while another kernel runs, it reports the shader clock that kernel
-// runs at (one clock domain for all compute units).  The loops end on the real-time counter and on an iteration cap.
+// and reads them again: launched on a second stream while another kernel runs, it reports the shader clock of the XCD
+// it lands on while that kernel runs (an indication, not a chip-wide average).  The loops end on the real-time counter
+// and on an iteration cap.
 __global__ __launch_bounds__(64) void clock_probe_kernel(uint64_t* counters, uint64_t delay_ticks, uint64_t window_ticks) {
     const uint64_t arrival = __builtin_amdgcn_s_memrealtime();
     for (uint32_t i = 0; i < (1u << 24) && __builtin_amdgcn_s_memrealtime() - arrival < delay_ticks; ++i) __builtin_amdgcn_s_sleep(64);
