@@ -277,6 +277,8 @@ extern "C" uint64_t khm_sliced_q_partial_output_stats_bytes(const khm_gqa_sdpa_c
 
 // ------------------------------------------------------------------------------------------ sliced-KV
 
+static int static_scratch_pointer(unsigned char** out);
+
 extern "C" int khm_sliced_kv_create(const khm_gqa_sdpa_config* config, const khm_sdpa_variant* variant,
                                     const khm_gqa_sdpa_shape* shape, khm_sliced_kv** out) {
     clear_error();
@@ -308,6 +310,10 @@ extern "C" int khm_sliced_kv_create(const khm_gqa_sdpa_config* config, const khm
         delete compute;
         return fail(KHM_ERR_UNSUPPORTED, "no gfx950 sliced-KV kernel for head_dim %u", config->head_dim);
     }
+    // Set-up is the place to look up this device's copy of the static scratch array (khm_sliced_kv_map_reduce_static),
+    // so that the entry point itself makes no runtime query on its first call.  Failing here is not an error of create.
+    unsigned char* static_scratch = nullptr;
+    if (static_scratch_pointer(&static_scratch) != KHM_OK) clear_error();
     *out = compute;
     return KHM_OK;
 }
@@ -421,7 +427,8 @@ constexpr uint64_t kStaticCounterBytes = 256ull << 10;   // arrival counters: a 
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 constexpr int kMaxDevices = 64;
-static unsigned char* static_scratch_of_device[kMaxDevices];   // filled on a device's first call; one stream user per handle, as everywhere here
+// filled when a compute is created on a device (else on the entry point's first call there); concurrent fills store the same value
+static unsigned char* static_scratch_of_device[kMaxDevices];
 
 __global__ __launch_bounds__(256) void clear_u32_kernel(uint32_t* words, uint32_t count) {
     const uint32_t index = blockIdx.x * 256 + threadIdx.x;
