@@ -93,12 +93,14 @@ static int build_q_token_ranges(const khm_request_shape* shapes, uint32_t num_re
 }
 
 // Greedy: repeatedly give one more split to the range whose splits are currently the longest
-// (ceil(iterations / splits)); ties go to the earlier range.
-static void allocate_kv_splits(std::vector<RangeWork>& ranges, uint32_t max_map_task_templates) {
+// (ceil(iterations / splits)); ties go to the earlier range.  `min_iterations_per_split` > 1 (the lookup route only)
+// keeps a range from being cut into splits shorter than that on average.
+static void allocate_kv_splits(std::vector<RangeWork>& ranges, uint32_t max_map_task_templates, uint32_t min_iterations_per_split = 1) {
     const size_t count = ranges.size();
     if (count == max_map_task_templates) return;
+    auto most_splits = [&](const RangeWork& range) { return std::max(range.num_kv_iterations / min_iterations_per_split, 1u); };
     if (count == 1) {
-        ranges[0].num_kv_splits = std::min(ranges[0].num_kv_iterations, max_map_task_templates);
+        ranges[0].num_kv_splits = std::min(most_splits(ranges[0]), max_map_task_templates);
         return;
     }
     struct Candidate {
@@ -111,7 +113,7 @@ static void allocate_kv_splits(std::vector<RangeWork>& ranges, uint32_t max_map_
     };
     std::priority_queue<Candidate> heap;
     for (size_t i = 0; i < count; ++i) {
-        if (ranges[i].num_kv_splits < ranges[i].num_kv_iterations)
+        if (ranges[i].num_kv_splits < most_splits(ranges[i]))
             heap.push(Candidate{div_ceil_u32(ranges[i].num_kv_iterations, ranges[i].num_kv_splits), i});
     }
     for (size_t used = count; used < max_map_task_templates; ++used) {
@@ -120,7 +122,7 @@ static void allocate_kv_splits(std::vector<RangeWork>& ranges, uint32_t max_map_
         heap.pop();
         RangeWork& range = ranges[top.index];
         range.num_kv_splits += 1;
-        if (range.num_kv_splits < range.num_kv_iterations)
+        if (range.num_kv_splits < most_splits(range))
             heap.push(Candidate{div_ceil_u32(range.num_kv_iterations, range.num_kv_splits), top.index});
     }
 }
@@ -129,7 +131,8 @@ static bool mul_u64(uint64_t a, uint64_t b, uint64_t* out) { return !__builtin_m
 
 static int materialize_candidate(const khm_selector& selector, const khm_sdpa_variant& variant, const khm_request_shape* shapes,
                                  uint32_t num_requests, const GqaReplayBucketPolicy& policy, uint32_t num_total_tokens,
-                                 bool has_slice, uint32_t kv_slice, bool direct_output, khm_selection* selection) {
+                                 bool has_slice, uint32_t kv_slice, bool direct_output, khm_selection* selection,
+                                 uint32_t split_budget = 0, uint32_t min_iterations_per_split = 1) {
     const khm_selector_limits& limits = selector.limits;
     const uint32_t max_q_tokens = variant.map_max_q_tokens;
     const uint32_t stage = variant.map_kv_tokens_per_iteration;
@@ -144,9 +147,11 @@ static int materialize_candidate(const khm_selector& selector, const khm_sdpa_va
         KHM_REQUIRE(total <= limits.max_map_task_templates, "GQA fixed slices exceed the Map task-template capacity");
     } else {
         uint32_t budget = limits.max_map_task_templates;
-        if (variant.map_kind != KHM_MAP_SLICED_KV && stage == 32)
+        if (split_budget != 0)
+            budget = std::min(std::max<uint32_t>(split_budget, (uint32_t)ranges.size()), limits.max_map_task_templates);
+        else if (variant.map_kind != KHM_MAP_SLICED_KV && stage == 32)
             budget = (uint32_t)std::min<uint64_t>((uint64_t)ranges.size() * 2, limits.max_map_task_templates);
-        allocate_kv_splits(ranges, budget);
+        allocate_kv_splits(ranges, budget, min_iterations_per_split);
     }
 
     selection->variant = variant;
@@ -281,9 +286,13 @@ static int validate_request_shapes(const khm_selector& selector, const khm_reque
 //       q * ratio <= 64  -> one sliced-Q tile of q tokens x ratio heads (verify blocks).
 //       q >= 16          -> dense prefill: the largest power-of-two token tile with tile * ratio <= 256 (128 at D 256).
 //       otherwise        -> the largest power-of-two token tile with tile * ratio <= 64.
-//   * KV slice.  A block streams its slice once, so slices only need to be short enough to fill the
-//     chip: aim for kTargetBlocks blocks in total, never below kMinSlice tokens (shorter slices pay
-//     more in partial traffic than they gain in parallelism), never above the longest context.
+//   * KV splits.  A block streams its split once, so splits only need to be short enough to fill the
+//     chip: kTargetBlocks blocks in total and not one more, because the verify kernels hold two (bf16 pages) or four
+//     (FP8 pages) blocks per compute unit and blocks beyond a whole number of rounds run in a nearly empty one (1448 blocks
+//     of a batch of 16 speculative requests took two rounds of 1024 slots on FP8 pages).  The template budget is handed
+//     out greedily, one more split at a time to the range whose splits are currently the longest, so all blocks end up
+//     about equally long, in whole 64-token iterations; a range is never cut into splits shorter than kMinSlice tokens on
+//     average (shorter ones pay more in partial traffic than they gain in parallelism).
 //     When the unsplit grid already has kTargetBlocks / 2 blocks, sliced-Q runs unsplit with direct output.
 // ---------------------------------------------------------------------------------------------
 constexpr uint64_t kTargetBlocks = 1024;
@@ -308,8 +317,10 @@ static int lookup_variant(const khm_sdpa_config& config, uint32_t queries, khm_s
     return khm_sdpa_variant_sliced_q(&config, KHM_MAP_Q_TOKENS_AND_HEADS, tile, 64, heads, out);
 }
 
+// Outputs: `direct` (one unsplit Map per Q range, final output) or else `split_budget`, the number of Map task templates
+// to hand out over the Q ranges.
 static int lookup_route(const khm_selector& selector, const khm_request_shape* shapes, uint32_t num_requests,
-                        khm_sdpa_variant* variant, uint32_t* slice, bool* direct) {
+                        khm_sdpa_variant* variant, uint32_t* slice, bool* direct, uint32_t* split_budget) {
     const khm_sdpa_config& config = selector.config;
     uint32_t max_q = 0, end = 0;
     for (uint32_t r = 0; r < num_requests; ++r) {
@@ -320,31 +331,20 @@ static int lookup_route(const khm_selector& selector, const khm_request_shape* s
     if (int status = lookup_variant(config, queries, variant)) return status;
     const uint64_t tile = variant->map_max_q_tokens;
     const uint64_t blocks_per_map = (uint64_t)config.num_kv_heads * div_ceil_u32(ratio_of(config), variant->map_max_q_heads);
-    // Work in (range, visible token) units, as the reference's capacity bound counts it (sdpa.rs:291-306).
-    uint64_t num_ranges = 0, visible = 0;
-    for (uint32_t r = 0; r < num_requests; ++r) {
-        const uint64_t q = shapes[r].num_q_tokens;
-        const uint64_t ranges = div_ceil_u64(q, tile);
-        num_ranges += ranges;
-        visible += ranges * shapes[r].num_history_tokens + tile * ranges * (ranges - 1) / 2 + q;
-    }
+    uint64_t num_ranges = 0;
+    for (uint32_t r = 0; r < num_requests; ++r) num_ranges += div_ceil_u64(shapes[r].num_q_tokens, tile);
     const bool can_direct = variant->map_kind != KHM_MAP_SLICED_KV;
     if (can_direct && (num_ranges * blocks_per_map >= kTargetBlocks / 2 || end <= kMinSlice)) {
         *slice = end;
         *direct = true;
         return KHM_OK;
     }
-    const uint64_t wanted_maps = std::max<uint64_t>(div_ceil_u64(kTargetBlocks, blocks_per_map), num_ranges);
-    uint64_t chosen = std::max<uint64_t>(visible / wanted_maps, 1);
-    chosen = 1ull << ilog2_u64(chosen);
-    chosen = std::max<uint64_t>(chosen, kMinSlice);
-    // Sum ceil(visible_i / slice) <= ceil(visible / slice) + ranges - 1 must fit the recorded capacity.
+    // a whole number of blocks per template: round the budget down so that the grid does not exceed kTargetBlocks
+    const uint64_t wanted_maps = std::max<uint64_t>(kTargetBlocks / blocks_per_map, num_ranges);
     KHM_REQUIRE(selector.limits.max_map_task_templates >= num_ranges, "GQA Q-token ranges exceed the Map task-template capacity");
-    const uint64_t split_budget = (uint64_t)selector.limits.max_map_task_templates - num_ranges + 1;
-    chosen = std::max(chosen, div_ceil_u64(visible, split_budget));
-    chosen = std::min<uint64_t>(chosen, end);
-    *slice = (uint32_t)chosen;
-    *direct = can_direct && chosen >= end;
+    *slice = end;
+    *direct = false;
+    *split_budget = (uint32_t)std::min<uint64_t>(wanted_maps, selector.limits.max_map_task_templates);
     return KHM_OK;
 }
 
@@ -355,10 +355,19 @@ static int select_impl(const khm_selector& selector, const khm_request_shape* sh
     const khm_sdpa_config& config = selector.config;
     if (selector.lookup) {
         khm_sdpa_variant variant;
-        uint32_t slice = 0;
+        uint32_t slice = 0, split_budget = 0;
         bool direct = false;
-        if (int status = lookup_route(selector, shapes, num_requests, &variant, &slice, &direct)) return status;
-        return materialize_candidate(selector, variant, shapes, num_requests, policy, num_total_tokens, true, slice, direct, result);
+        if (int status = lookup_route(selector, shapes, num_requests, &variant, &slice, &direct, &split_budget)) return status;
+        if (direct)
+            return materialize_candidate(selector, variant, shapes, num_requests, policy, num_total_tokens, true, slice, true, result);
+        const uint32_t min_iterations = std::max(kMinSlice / variant.map_kv_tokens_per_iteration, 1u);
+        if (int status = materialize_candidate(selector, variant, shapes, num_requests, policy, num_total_tokens, false, 0, false,
+                                               result, split_budget, min_iterations))
+            return status;
+        // nothing was split (short contexts): sliced-Q then writes its output directly, no Reduce
+        if (variant.map_kind != KHM_MAP_SLICED_KV && result->map_task_templates.size() == result->q_token_ranges.size())
+            return materialize_candidate(selector, variant, shapes, num_requests, policy, num_total_tokens, true, slice, true, result);
+        return KHM_OK;
     }
     auto materialize = [&](const khm_sdpa_variant& variant, khm_selection* out) {
         return materialize_candidate(selector, variant, shapes, num_requests, policy, num_total_tokens, false, 0, false, out);
