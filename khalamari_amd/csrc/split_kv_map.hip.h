@@ -47,7 +47,7 @@ struct KvTile {
     uint32_t first_token;
 };
 
-template <int D, int NT, int NWAVES>
+template <int D, int NT, int NWAVES, bool Q_IN_LDS = (NT != 1)>
 struct MapSmem {
     static constexpr int kVRowBytes = D * 2 + 32;          // +32 B: rows 8 banks apart, conflict-free transposed reads
     static constexpr int kVBytes = NWAVES * 16 * kVRowBytes;
@@ -58,7 +58,7 @@ struct MapSmem {
     static constexpr int kOBytes = (kTilePerWave ? NWAVES : 1) * kCols * kORowFloats * 4;
     static constexpr int kUnionBytes = kVBytes > kOBytes ? kVBytes : kOBytes;
     static constexpr int kQRowBytes = D * 2 + 16;
-    static constexpr int kQBytes = NT == 1 ? 0 : kCols * kQRowBytes;   // a single column tile keeps Q in registers
+    static constexpr int kQBytes = Q_IN_LDS ? kCols * kQRowBytes : 0;   // a single column tile keeps Q in registers
     static constexpr int kStatsBytes = (NWAVES + 1) * kCols * 3 * 4;   // (reference, sum, maximum) per wave and column
     static constexpr int kTotal = kUnionBytes + kQBytes + kStatsBytes;
 };
@@ -78,8 +78,14 @@ __global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapPara
     constexpr int LOADS = KvTile<D, KV8>::kLoads;
     // first dim of the eight that lane group g contracts in k-step ks (the K fragments above fix the order)
     auto q_dim = [](int ks, int g) { return KV8 ? (ks >> 1) * 64 + g * 16 + (ks & 1) * 8 : ks * 32 + g * 8; };
-    using Smem = MapSmem<D, NT, NWAVES>;
-    constexpr bool kQInRegs = (NT == 1);
+    // D 256 on FP8 pages: with the Q fragments read from LDS and one tile requested ahead instead of two the kernel takes
+    // 236 registers instead of 296, so a compute unit holds two blocks (two waves per SIMD) instead of one; these blocks
+    // run at the pace of their own load -> decode -> MFMA chain, which a second wave on the SIMD overlaps (four requests of
+    // 131072 tokens: 200 -> 194 us).  bf16 pages at D 256 stay at one block either way (399 registers) and are within 3 %
+    // of a read-only launch; at D 128 a third block per CU was measured and changes nothing.
+    constexpr bool kSlim = D == 256 && KV8;
+    constexpr bool kQInRegs = (NT == 1) && !kSlim;
+    using Smem = MapSmem<D, NT, NWAVES, !kQInRegs>;
 
     __shared__ __align__(16) unsigned char smem[Smem::kTotal];
     unsigned char* v_lds_all = smem;
@@ -443,7 +449,7 @@ __global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapPara
     // ---- main loop: a ring of register buffers, loads DEPTH tiles ahead ----------------------
     // Two tiles in flight per wave (8 KB each at D 128 on bf16 pages, half that on FP8 pages, where four in flight were
     // measured slower than two).  The ring is indexed with compile-time constants after unrolling.
-    constexpr int DEPTH = kMapPrefetchDepth;
+    constexpr int DEPTH = kSlim ? 1 : kMapPrefetchDepth;
     if (num_wave_tiles > 0) {
         KvTile<D, KV8> ring[DEPTH + 1];
 #pragma unroll

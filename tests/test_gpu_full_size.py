@@ -59,7 +59,7 @@ def _run_step(workload, pool_index=0):
     return gpu_runner.bf16_tensor_to_f32(workload.out.view(torch.int16))
 
 
-@pytest.mark.parametrize("index,fp8", [(1, False), (2, False), (2, True), (3, False)])
+@pytest.mark.parametrize("index,fp8", [(1, False), (2, False), (2, True), (3, False), (3, True)])
 def test_decode_configs_at_full_size(device, index, fp8):
     workload = bench.Workload(index, device, num_pools=1, fp8_pages=fp8)
     actual = _run_step(workload)
