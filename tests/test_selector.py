@@ -323,3 +323,25 @@ def test_lookup_fills_the_chip_for_the_benchmark_shapes():
     policy = GQAReplayBucketPolicy(16384, prefill.limits().max_map_task_templates)
     result = selector_prefill.select([RequestShape(4096, 2048)] * 8, policy, 16384)
     assert result.direct_output()
+
+
+def test_lookup_hands_out_exactly_the_block_budget_in_equal_splits():
+    """A batch of 16 speculative blocks (q_len 2..5 on contexts of 4096..32768 tokens, Hq64/Hkv8): the verify kernels hold a
+    whole number of blocks per compute unit, so the route must not exceed 1024 blocks, and the splits of all ranges end up
+    about equally long, in whole 64-token iterations."""
+    config = _cfg(64, 8, 128, 16)
+    histories = [4096 + 1791 * i for i in range(16)]
+    q_lens = [2 + i % 4 for i in range(16)]
+    selector = Selector.for_lookup(config, sum(q_lens), Layout(16, 1, 2064, 1))
+    policy = GQAReplayBucketPolicy(selector.limits().max_tokens, selector.limits().max_map_task_templates)
+    result = selector.select([RequestShape(h, q) for h, q in zip(histories, q_lens)], policy, sum(q_lens))
+    templates = result.map_task_templates()
+    assert not result.direct_output()
+    assert len(templates) * 8 == 1024
+    lengths = [end - begin for (_, begin, end) in templates]
+    assert max(lengths) <= 2 * min(lengths) and min(lengths) >= 256
+    assert all(begin % 64 == 0 for (_, begin, _) in templates)
+    _assert_contiguous_cover(result)
+    # short contexts are not cut below 256 tokens per split on average, and an unsplit sliced-Q batch writes its output directly
+    short = selector.select([RequestShape(300, 3)] * 4, policy, 12)
+    assert short.direct_output() and len(short.map_task_templates()) == len(short.q_token_ranges())
