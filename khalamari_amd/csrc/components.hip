@@ -58,8 +58,8 @@ static TileKernelChoice select_tile_kernel(uint32_t head_dim, uint32_t coordinat
             if (wide) return {tile_map_kernel<128, 2, 8, 64, 4, 1, true, true>, 512, (uint32_t)TileSmem<128, 64, 4>::kBytes};
             return {tile_map_kernel<128, 2, 4, 64, 4, 2, true, true>, 256, (uint32_t)TileSmem<128, 64, 4>::kBytes};
         }
-        if (wide) return {tile_map_kernel<128, 2, 8, 64, 4, 1, false, true>, 512, (uint32_t)TileSmem<128, 64, 4>::kBytes};
-        return {tile_map_kernel<128, 1, 8, 32, 4, 2, false, true>, 512, (uint32_t)TileSmem<128, 32, 4>::kBytes};
+        if (wide) return {tile_map_kernel<128, 2, 8, 64, 4, 1, false, true>, 512, (uint32_t)TileSmem<128, 64, 4, 256, true>::kBytes};
+        return {tile_map_kernel<128, 1, 8, 32, 4, 2, false, true>, 512, (uint32_t)TileSmem<128, 32, 4, 256, true>::kBytes};
     }
     if (kv_dtype == KHM_DTYPE_FP8_E4M3FN) {
         if (head_dim == 128) {
@@ -78,13 +78,13 @@ static TileKernelChoice select_tile_kernel(uint32_t head_dim, uint32_t coordinat
     }
     if (head_dim == 128) {
         if (coordinates <= 64)
-            return {tile_map_kernel<128, 1, 4, 32, 4, 2>, 256, (uint32_t)TileSmem<128, 32, 4>::kBytes};  // 64 KB: two blocks per CU
+            return {tile_map_kernel<128, 1, 4, 32, 4, 2>, 256, (uint32_t)TileSmem<128, 32, 4, 256, true>::kBytes};  // 64 KB: two blocks per CU
         // 65..128 coordinates on bf16 pages: eight waves of one column tile each, BK 32, 64 KB of LDS, two blocks per CU =
         // four waves per SIMD at 118 VGPRs.  A batch of 2048-token chunks held to 128 columns: 5.13 ms, against 6.93 ms
         // on four waves of two column tiles with BK 64 (and 5.77 ms on eight waves with BK 64 at one block per CU).  FP8
         // pages keep the four-wave tile: a 32-token FP8 tile has fewer load units than eight waves.
-        if (coordinates <= 128) return {tile_map_kernel<128, 1, 8, 32, 4, 2>, 512, (uint32_t)TileSmem<128, 32, 4>::kBytes};
-        return {tile_map_kernel<128, 2, 8, 64, 4, 1>, 512, (uint32_t)TileSmem<128, 64, 4>::kBytes};
+        if (coordinates <= 128) return {tile_map_kernel<128, 1, 8, 32, 4, 2>, 512, (uint32_t)TileSmem<128, 32, 4, 256, true>::kBytes};
+        return {tile_map_kernel<128, 2, 8, 64, 4, 1>, 512, (uint32_t)TileSmem<128, 64, 4, 256, true>::kBytes};
     }
     if (head_dim == 256) {
         // 65..128 coordinates: eight waves of one column tile each (167 VGPRs, two waves per SIMD) rather than four waves

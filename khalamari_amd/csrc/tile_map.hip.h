@@ -30,12 +30,28 @@
 
 namespace khm {
 
-template <int D, int BK, int NSTAGES, int ROW_BYTES = D * 2>
+// LDS tiles.  A tile is made of units: the 1024 bytes one wave load (64 lanes x 16 bytes) delivers, which the loading
+// lanes may fill with any 64 of the 16-byte chunks of the rows the unit covers.
+// LINEAR (bf16 pages at head dim 128, rows of 256 bytes, four rows per unit): every fragment a lane reads during a slice
+// sits at a fixed distance from the lane's first one, so the reads of a slice share one address register and differ in
+// their immediate offsets only.  A unit holds its rows in pieces of 64 bytes, piece q of row r at 256 q + 64 r, which
+// keeps four neighbouring lanes of a wave load on 64 contiguous bytes of a page; inside a K piece the four chunks are
+// XORed with the unit index, and V units lie 1056 bytes apart, so that the lanes the LDS serves together (sixteen
+// rows of a K read, two units of a transposed V read) fall on different banks.
+// Other tiles keep rows whole and XOR the chunk index with the row (see the swizzles in the kernel).
+template <int D, int BK, int NSTAGES, int ROW_BYTES = D * 2, bool LINEAR = false>
 struct TileSmem {
+    static_assert(!LINEAR || ROW_BYTES == 256, "the linear layout is written for rows of 256 bytes");
     static constexpr int kRowBytes = ROW_BYTES;
-    static constexpr int kTileBytes = BK * kRowBytes;
-    static constexpr int kBytes = 2 /*K,V*/ * NSTAGES * kTileBytes;
+    static constexpr int kRowsPerUnit = 1024 / ROW_BYTES;
+    static constexpr int kUnitsPerTile = BK / kRowsPerUnit;
+    static constexpr int kVUnitPitch = LINEAR ? 1056 : 1024;
+    static constexpr int kKTileBytes = BK * kRowBytes;
+    static constexpr int kVTileBytes = kUnitsPerTile * kVUnitPitch;
+    static constexpr int kBytes = NSTAGES * (kKTileBytes + kVTileBytes);
 };
+// which kernels use the linear layout (the host sizes the dynamic LDS with the same rule)
+constexpr bool tile_layout_is_linear(int head_dim, bool fp8_pages) { return head_dim == 128 && !fp8_pages; }
 
 
 // 16 bytes per lane from global memory to LDS: lane l of the wave reads uniform_base + lane_offset and lands at
@@ -96,17 +112,38 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     constexpr bool RAW8 = KV8 && NTW == 1 && NWAVES == 4;   // raw FP8 codes in LDS, decoded by the waves that read them
     constexpr bool STAGED8 = KV8 && !RAW8;       // FP8 tiles decoded once on their way into bf16 LDS tiles
     static_assert(!STAGED8 || NSTAGES == 4, "the register-staged FP8 path is written for a ring of four tiles");
-    using Smem = TileSmem<D, BK, NSTAGES, RAW8 ? D : 2 * D>;
+    constexpr bool LINEAR = tile_layout_is_linear(D, KV8);
+    using Smem = TileSmem<D, BK, NSTAGES, RAW8 ? D : 2 * D, LINEAR>;
     constexpr int ROW = Smem::kRowBytes;
+    constexpr int V_UNIT = Smem::kVUnitPitch;
     // XOR swizzle of the 16-byte chunk position inside an LDS row, by tile row.  bf16 rows (and raw rows of 256 bytes)
     // alias bank for bank, so K reads spread sixteen rows over sixteen positions and the transposed V reads eight rows
     // over every second one; raw rows of 128 bytes alias in pairs and have eight chunks: both planes use (row / 2) % 8.
     auto k_swizzle_of = [](uint32_t row) -> uint32_t { return (RAW8 && D == 128) ? ((row >> 1) & 7u) : (row & 15u); };
     auto v_swizzle_of = [](uint32_t row) -> uint32_t { return RAW8 ? (D == 128 ? ((row >> 1) & 7u) : (row & 15u)) : ((row & 7u) << 1); };
+    // Where chunk `chunk` (16 bytes) of tile row `row` sits inside its K or V tile in LDS.
+    auto k_place = [&](uint32_t row, uint32_t chunk) -> uint32_t {
+        if constexpr (LINEAR) return (row >> 2) * 1024 + (chunk >> 2) * 256 + ((row & 3u) << 6) + ((((0u - chunk) ^ (row >> 2)) & 3u) << 4);
+        else return row * ROW + ((chunk ^ k_swizzle_of(row)) << 4);
+    };
+    auto v_place = [&](uint32_t row, uint32_t chunk) -> uint32_t {
+        if constexpr (LINEAR) return (row >> 2) * V_UNIT + (chunk >> 2) * 256 + ((row & 3u) << 6) + ((chunk & 3u) << 4);
+        else return row * ROW + ((chunk ^ v_swizzle_of(row)) << 4);
+    };
+    // The inverse, for the lane that fills 16-byte slot `slot` of unit `unit` of a tile: row inside the tile and chunk.
+    struct Source { uint32_t row, chunk; };
+    auto k_source_of = [&](uint32_t unit, uint32_t slot) -> Source {
+        if constexpr (LINEAR) return Source{unit * 4 + ((slot >> 2) & 3u), (slot >> 4) * 4 + ((0u - (slot ^ unit)) & 3u)};
+        else { const uint32_t row = unit * RPL + slot / CPR; return Source{row, (slot % CPR) ^ k_swizzle_of(row)}; }
+    };
+    auto v_source_of = [&](uint32_t unit, uint32_t slot) -> Source {
+        if constexpr (LINEAR) return Source{unit * 4 + ((slot >> 2) & 3u), (slot >> 4) * 4 + (slot & 3u)};
+        else { const uint32_t row = unit * RPL + slot / CPR; return Source{row, (slot % CPR) ^ v_swizzle_of(row)}; }
+    };
 
     extern __shared__ __align__(1024) unsigned char tile_smem[];
     unsigned char* k_lds = tile_smem;                                    // [NSTAGES][BK][ROW]
-    unsigned char* v_lds = tile_smem + NSTAGES * Smem::kTileBytes;       // [NSTAGES][BK][ROW]
+    unsigned char* v_lds = tile_smem + NSTAGES * Smem::kKTileBytes;      // [NSTAGES][units][V_UNIT]
     const uint32_t k_lds_address = lds_address_of(k_lds);
     const uint32_t v_lds_address = lds_address_of(v_lds);
 
@@ -306,16 +343,12 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     // Lane offsets of a wave load inside its page.  A tile that lies wholly inside [blk_lo, blk_hi) needs no clamp and,
     // BK being a multiple of the page size, its offsets do not depend on the tile: those live in registers.
     uint32_t k_lane_offset[UPW], v_lane_offset[UPW];
-    {
-        const uint32_t load_row = lane / CPR;       // row inside a wave load
-        const uint32_t load_pos = lane % CPR;       // 16-byte position inside the row
 #pragma unroll
-        for (int i = 0; i < UPW; ++i) {
-            const uint32_t row = (wave * UPW + i) * RPL + load_row;                // row inside the tile
-            const uint32_t in_page = ((first_token + row) & (tpp - 1)) * PAGE_ROW;
-            k_lane_offset[i] = in_page + ((load_pos ^ k_swizzle_of(row)) << 4);
-            v_lane_offset[i] = in_page + ((load_pos ^ v_swizzle_of(row)) << 4);
-        }
+    for (int i = 0; i < UPW; ++i) {
+        const Source k_source = k_source_of(wave * UPW + i, lane), v_source = v_source_of(wave * UPW + i, lane);
+        k_lane_offset[i] = ((first_token + k_source.row) & (tpp - 1)) * PAGE_ROW + (k_source.chunk << 4);
+        // K and V of a wave load share one scalar base (the K plane of their page): the V offsets carry the distance
+        v_lane_offset[i] = ((first_token + v_source.row) & (tpp - 1)) * PAGE_ROW + (v_source.chunk << 4) + (uint32_t)(plane_v - plane_k);
     }
     auto issue_tile = [&](uint32_t tile, const TileIds ids) __attribute__((always_inline)) {
         const uint32_t stage = tile % NSTAGES;
@@ -324,28 +357,49 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
 #pragma unroll
             for (int i = 0; i < UPW; ++i) {
                 const uint32_t unit = wave * UPW + i;                                  // wave-uniform
-                const unsigned char* page = p.kv_pages + (uint64_t)ids[i] * p.page_bytes;   // scalar
-                load_to_lds_b128(page + plane_k, k_lane_offset[i], k_lds_address + stage * Smem::kTileBytes + unit * 1024);
-                load_to_lds_b128(page + plane_v, v_lane_offset[i], v_lds_address + stage * Smem::kTileBytes + unit * 1024);
+                const unsigned char* page = p.kv_pages + plane_k + (uint64_t)ids[i] * p.page_bytes;   // scalar
+                load_to_lds_b128(page, k_lane_offset[i], k_lds_address + stage * Smem::kKTileBytes + unit * 1024);
+                load_to_lds_b128(page, v_lane_offset[i], v_lds_address + stage * Smem::kVTileBytes + unit * V_UNIT);
             }
             return;
         }
         // first or last tile of the range: rows outside it are redirected, which changes their offsets
-        const uint32_t load_row = lane / CPR;
-        const uint32_t load_pos = lane % CPR;
 #pragma unroll
         for (int i = 0; i < UPW; ++i) {
             const uint32_t unit = wave * UPW + i;
-            const uint32_t row = unit * RPL + load_row;
-            uint32_t token = tile_token + row;
-            token = token < blk_lo ? blk_lo : token;
-            token = token >= blk_hi ? blk_hi - 1 : token;
+            const Source k_source = k_source_of(unit, lane), v_source = v_source_of(unit, lane);
+            auto in_page_of = [&](uint32_t row) {
+                uint32_t token = tile_token + row;
+                token = token < blk_lo ? blk_lo : token;
+                token = token >= blk_hi ? blk_hi - 1 : token;
+                return (token & (tpp - 1)) * PAGE_ROW;
+            };
             const unsigned char* page = p.kv_pages + (uint64_t)ids[i] * p.page_bytes;
-            const uint32_t in_page = (token & (tpp - 1)) * PAGE_ROW;
-            const uint32_t k_offset_bytes = in_page + ((load_pos ^ k_swizzle_of(row)) << 4);
-            const uint32_t v_offset_bytes = in_page + ((load_pos ^ v_swizzle_of(row)) << 4);
-            load_to_lds_b128(page + plane_k, k_offset_bytes, k_lds_address + stage * Smem::kTileBytes + unit * 1024);
-            load_to_lds_b128(page + plane_v, v_offset_bytes, v_lds_address + stage * Smem::kTileBytes + unit * 1024);
+            load_to_lds_b128(page + plane_k, in_page_of(k_source.row) + (k_source.chunk << 4), k_lds_address + stage * Smem::kKTileBytes + unit * 1024);
+            load_to_lds_b128(page + plane_v, in_page_of(v_source.row) + (v_source.chunk << 4), v_lds_address + stage * Smem::kVTileBytes + unit * V_UNIT);
+        }
+    };
+
+    // The same two steps for a tile known to lie wholly inside [blk_lo, blk_hi), as the steady-state loop requests them:
+    // no clamps, no branches.
+    auto fetch_ids_interior = [&](uint32_t tile) __attribute__((always_inline)) -> TileIds {
+        TileIds ids;
+        const uint32_t last_page = p.pages_per_request_layer - 1;
+#pragma unroll
+        for (int i = 0; i < UPW; ++i) {
+            const uint32_t page = (first_token + tile * BK + (wave * UPW + i) * RPL) >> tpp_shift;
+            ids[i] = load_uniform_u32(table, page < last_page ? page : last_page);   // the tile after the last one requested is read, not used
+        }
+        return ids;
+    };
+    const unsigned char* const k_plane_base = p.kv_pages + plane_k;
+    auto issue_interior_tile = [&](uint32_t stage, const TileIds ids) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < UPW; ++i) {
+            const uint32_t unit = wave * UPW + i;
+            const unsigned char* page = k_plane_base + (uint64_t)ids[i] * p.page_bytes;
+            load_to_lds_b128(page, k_lane_offset[i], k_lds_address + stage * Smem::kKTileBytes + unit * 1024);
+            load_to_lds_b128(page, v_lane_offset[i], v_lds_address + stage * Smem::kVTileBytes + unit * V_UNIT);
         }
     };
 
@@ -370,18 +424,17 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     auto write_raw_tile = [&](uint32_t tile) __attribute__((always_inline)) {
         const uint32_t load_row = lane / CPR;
         const uint32_t load_pos = lane % CPR;
-        unsigned char* k_stage = k_lds + (tile % NSTAGES) * Smem::kTileBytes;
-        unsigned char* v_stage = v_lds + (tile % NSTAGES) * Smem::kTileBytes;
+        unsigned char* k_stage = k_lds + (tile % NSTAGES) * Smem::kKTileBytes;
+        unsigned char* v_stage = v_lds + (tile % NSTAGES) * Smem::kVTileBytes;
 #pragma unroll
         for (int i = 0; i < UPW; ++i) {
             const uint32_t row = (wave * UPW + i) * RPL + load_row;
-            const uint32_t k_swizzle = row & 15, v_swizzle_row = (row & 7) << 1;
             const uint4 k_low = fp8x8_to_bf16x8(make_uint2(raw_k[i].x, raw_k[i].y)), k_high = fp8x8_to_bf16x8(make_uint2(raw_k[i].z, raw_k[i].w));
             const uint4 v_low = fp8x8_to_bf16x8(make_uint2(raw_v[i].x, raw_v[i].y)), v_high = fp8x8_to_bf16x8(make_uint2(raw_v[i].z, raw_v[i].w));
-            *reinterpret_cast<uint4*>(k_stage + row * ROW + (((2 * load_pos) ^ k_swizzle) << 4)) = k_low;
-            *reinterpret_cast<uint4*>(k_stage + row * ROW + (((2 * load_pos + 1) ^ k_swizzle) << 4)) = k_high;
-            *reinterpret_cast<uint4*>(v_stage + row * ROW + (((2 * load_pos) ^ v_swizzle_row) << 4)) = v_low;
-            *reinterpret_cast<uint4*>(v_stage + row * ROW + (((2 * load_pos + 1) ^ v_swizzle_row) << 4)) = v_high;
+            *reinterpret_cast<uint4*>(k_stage + k_place(row, 2 * load_pos)) = k_low;
+            *reinterpret_cast<uint4*>(k_stage + k_place(row, 2 * load_pos + 1)) = k_high;
+            *reinterpret_cast<uint4*>(v_stage + v_place(row, 2 * load_pos)) = v_low;
+            *reinterpret_cast<uint4*>(v_stage + v_place(row, 2 * load_pos + 1)) = v_high;
         }
     };
 
@@ -393,7 +446,7 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         if constexpr (RAW8) k_offset[ks] = r16 * ROW + ((((uint32_t)ks * 2 + (g >> 1)) ^ k_swizzle_of(r16)) << 4) + (g & 1) * 8;
-        else k_offset[ks] = r16 * ROW + (((ks * 4 + g) ^ r16) << 4);
+        else k_offset[ks] = k_place(r16, ks * 4 + g);   // layouts with fixed distances: k_offset[0] + 256 * ks
     }
     // V: lane (g, r) passes row 4g + r/4 (+16 for the second half), dims mt*16 + 4*(r%4) .. +3, i.e. source chunk
     // 2*mt + (r%4)/2, stored at position chunk ^ 2*(row & 7).
@@ -403,7 +456,8 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     // weights it holds, in their order.
     const uint32_t v_row = RAW8 ? ((r16 >> 1) < 4 ? g * 4 + (r16 >> 1) : 16 + g * 4 + (r16 >> 1) - 4) : g * 4 + (r16 >> 2);
     const uint32_t v_swizzle = RAW8 ? v_swizzle_of(v_row) : ((r16 & 3) >> 1) ^ ((v_row & 7) << 1);
-    const uint32_t v_base = v_row * ROW + (r16 & 1) * 8;
+    const uint32_t v_base = LINEAR ? v_place(v_row, (r16 & 3) >> 1) + (r16 & 1) * 8 : v_row * ROW + (r16 & 1) * 8;
+    constexpr uint32_t kSixteenRows = LINEAR ? 4 * V_UNIT : 16 * ROW;   // V rows 16 apart in a tile
     auto v_fragment = [&](const unsigned char* v_src, int mt) __attribute__((always_inline)) -> bf16x8 {
         if constexpr (RAW8) {
             typedef int CodeWords __attribute__((ext_vector_type(2)));
@@ -411,9 +465,9 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             const CodeWords codes = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CodeWords __attribute__((address_space(3)))*)(address));
             return __builtin_bit_cast(bf16x8, fp8x8_to_bf16x8(make_uint2((uint32_t)codes[0], (uint32_t)codes[1])));
         } else {
-            const unsigned char* address = v_src + v_base + (((mt * 2) ^ v_swizzle) << 4);
+            const unsigned char* address = v_src + v_base + (LINEAR ? (uint32_t)((mt >> 1) * 256 + (mt & 1) * 32) : ((mt * 2) ^ v_swizzle) << 4);
             const uint2 lo = __builtin_bit_cast(uint2, lds_read_tr16(address));
-            const uint2 hi = __builtin_bit_cast(uint2, lds_read_tr16(address + 16 * ROW));
+            const uint2 hi = __builtin_bit_cast(uint2, lds_read_tr16(address + kSixteenRows));
             return __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
         }
     };
@@ -479,7 +533,8 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         // UNTRACKED: the largest score is not followed (direct output needs no partial state).  The weights are computed
         // straight away and the lane's sum of them, which the slice needs anyway, tells whether a score ran away from
         // the reference: one compare per column tile instead of a maximum over the lane's eight scores.
-        constexpr bool UNTRACKED = decltype(untracked_tag)::value;
+        constexpr bool UNTRACKED = decltype(untracked_tag)::value != 0;
+        constexpr bool ANCHORED = decltype(untracked_tag)::value == 2;   // untracked, and every column has its reference
         static_assert(!UNTRACKED || (!PRECISE && !MASKED), "the untracked slice is the plain interior one");
         Scores next;
         scores_of(k_next, next);
@@ -491,19 +546,18 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             auto weights = [&]() __attribute__((always_inline)) {
 #pragma unroll
                 for (int nt = 0; nt < NTW; ++nt) {
-                    slice_sum[nt] = 0.0f;
 #pragma unroll
                     for (int rt = 0; rt < 2; ++rt) {
                         float e[4];
 #pragma unroll
                         for (int i = 0; i < 4; ++i) e[i] = fast_exp2(s[rt][nt][i]);
-                        slice_sum[nt] += (e[0] + e[1]) + (e[2] + e[3]);
                         p_bits[nt][2 * rt] = pack_bf16x2(e[0], e[1]);
                         p_bits[nt][2 * rt + 1] = pack_bf16x2(e[2], e[3]);
+                        const float half_sum = (e[0] + e[1]) + (e[2] + e[3]);
+                        slice_sum[nt] = rt == 0 ? half_sum : slice_sum[nt] + half_sum;
                     }
                 }
             };
-            bool lane_wants_move = unanchored;
             auto relative_scores = [&]() __attribute__((always_inline)) {
 #pragma unroll
                 for (int nt = 0; nt < NTW; ++nt)
@@ -514,8 +568,11 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             };
             relative_scores();
             weights();
+            float largest_sum = slice_sum[0];
 #pragma unroll
-            for (int nt = 0; nt < NTW; ++nt) lane_wants_move = lane_wants_move | !(slice_sum[nt] <= kSumTrigger);
+            for (int nt = 1; nt < NTW; ++nt) largest_sum = fmaxf(largest_sum, slice_sum[nt]);
+            bool lane_wants_move = !(largest_sum <= kSumTrigger);
+            if constexpr (!ANCHORED) lane_wants_move = lane_wants_move | unanchored;
             if (__builtin_amdgcn_ballot_w64(lane_wants_move) != 0) {
                 // rare: some lane's weights add up to more than kSumTrigger (one of its scores is then more than
                 // kUntrackedMove above the reference), or a column has no reference yet.  The scores are computed again
@@ -599,7 +656,8 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
                     float e[4];
     #pragma unroll
                     for (int i = 0; i < 4; ++i) e[i] = fast_exp2(s[rt][nt][i]);
-                    slice_sum += (e[0] + e[1]) + (e[2] + e[3]);
+                    const float half_sum = (e[0] + e[1]) + (e[2] + e[3]);
+                    slice_sum = rt == 0 ? half_sum : slice_sum + half_sum;
                     p_bits[nt][2 * rt] = pack_bf16x2(e[0], e[1]);
                     p_bits[nt][2 * rt + 1] = pack_bf16x2(e[2], e[3]);
                     if constexpr (PRECISE) {
@@ -641,10 +699,10 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         else wait_vmem_outstanding<0>();
     };
     auto k_slice = [&](uint32_t slice) __attribute__((always_inline)) -> const unsigned char* {
-        return k_lds + ((slice / SL) % NSTAGES) * Smem::kTileBytes + (slice % SL) * 32 * ROW;
+        return k_lds + ((slice / SL) % NSTAGES) * Smem::kKTileBytes + (slice % SL) * 32 * ROW;
     };
     auto v_slice = [&](uint32_t slice) __attribute__((always_inline)) -> const unsigned char* {
-        return v_lds + ((slice / SL) % NSTAGES) * Smem::kTileBytes + (slice % SL) * 32 * ROW;
+        return v_lds + ((slice / SL) % NSTAGES) * Smem::kVTileBytes + (slice % SL) * (Smem::kVTileBytes / SL);
     };
     Scores pending;
     TileIds upcoming = fetch_ids(NSTAGES - 1);
@@ -700,6 +758,30 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             }
         }
     };
+    // Steady state of an interior run (direct loads, two slices per tile, untracked weights): every tile of
+    // [tile_begin, tile_end) has its successor's first slice in the range, and the tile NSTAGES - 1 ahead exists and lies
+    // wholly inside the block's KV range.  One straight-line body per tile: a fixed wait, the barrier, unconditional
+    // requests; the compiler is free to mix the S^T of the next slice with the softmax of this one.
+    auto run_steady_tiles = [&](uint32_t tile_begin, uint32_t tile_end) __attribute__((always_inline)) {
+        constexpr std::false_type no{};
+        constexpr std::integral_constant<int, 2> untracked_anchored{};
+        TileIds ahead = fetch_ids_interior(tile_begin + NSTAGES - 1);
+        for (uint32_t tile = tile_begin; tile < tile_end; ++tile) {
+            wait_vmem_outstanding<(NSTAGES - 3) * LPW>();   // tile + 1 has landed; tiles up to tile + NSTAGES - 2 are requested
+            barrier_keeping_loads_in_flight();
+            const uint32_t stage = tile % NSTAGES, next_stage = (tile + 1) % NSTAGES, free_stage = (tile + NSTAGES - 1) % NSTAGES;
+            const unsigned char* k_tile = k_lds + stage * Smem::kKTileBytes;
+            const unsigned char* v_tile = v_lds + stage * Smem::kVTileBytes;
+            auto request_next = [&]() __attribute__((always_inline)) {
+                issue_interior_tile(free_stage, ahead);
+                ahead = fetch_ids_interior(tile + NSTAGES);
+            };
+            auto nothing = []() __attribute__((always_inline)) {};
+            process_slice(no, no, untracked_anchored, 0u, pending, k_tile, k_tile + 32 * ROW, v_tile, request_next);
+            process_slice(no, no, untracked_anchored, 0u, pending, k_tile + 32 * ROW, k_lds + next_stage * Smem::kKTileBytes, v_tile + Smem::kVTileBytes / 2, nothing);
+        }
+    };
+
     if (num_tiles > 0) {
         if constexpr (STAGED8) {
             // tiles 0 and 1 into LDS, tile 2 into registers
@@ -760,7 +842,27 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
                 // no partial state to hand on: the interior slices need not follow the largest score
 #pragma unroll
                 for (int nt = 0; nt < NTW; ++nt) unanchored = unanchored | (lane_top[nt] == -INFINITY);
-                run_tiles(no, no, yes, head_end, tail_begin);
+                uint32_t steady_end = head_end;
+                if constexpr (!STAGED8 && SL == 2) {
+                    // tiles t with t + NSTAGES - 1 a whole tile inside [blk_lo, blk_hi): (t + NSTAGES) * BK <= blk_hi - first_token
+                    const uint32_t whole_tiles = (blk_hi - first_token) / BK;
+                    uint32_t limit = whole_tiles >= (uint32_t)NSTAGES ? whole_tiles - (NSTAGES - 1) : 0;
+                    limit = limit < tail_begin ? limit : tail_begin;
+                    if (limit > head_end) {
+                        uint32_t steady_begin = head_end;
+                        if (__builtin_amdgcn_ballot_w64(unanchored) != 0) {
+                            // a column without a reference yet: the general slice anchors it
+                            run_tiles(no, no, yes, head_end, head_end + 1);
+                            steady_begin = head_end + 1;
+                        }
+                        steady_end = limit;
+                        if (steady_end > steady_begin) {
+                            run_steady_tiles(steady_begin, steady_end);
+                            upcoming = fetch_ids(steady_end + NSTAGES - 1);
+                        }
+                    }
+                }
+                run_tiles(no, no, yes, steady_end, tail_begin);
             } else {
                 run_tiles(no, no, no, head_end, tail_begin);
             }

@@ -377,6 +377,23 @@ def test_chunked_prefill_onto_a_paged_prefix(device, hq, hkv, d, tile):
         helpers.assert_parity(actual, expected, f"prefill tile={tile} slice={kv_slice} direct={direct}")
 
 
+@pytest.mark.parametrize("hq,hkv,d,tile", [(16, 2, 128, 32), (8, 2, 128, 32)])
+def test_long_interior_runs_of_a_prefill_tile_checked_on_every_row(device, hq, hkv, d, tile):
+    """Prefixes of several thousand keys, so that nearly all tiles of a block are interior ones that run in the
+    steady-state loop of the direct-output builds (unconditional requests, weights that do not follow the largest
+    score); every Q row is compared with the oracle, at prefixes that start the KV walk on and off a tile boundary."""
+    histories = [5000, 1531, 4096]
+    q_lens = [96, 70, 33]
+    w = helpers.make_workload(num_q_heads=hq, num_kv_heads=hkv, head_dim=d, tokens_per_page=16, histories=histories,
+                              q_lens=q_lens, seed=411, garbage_bits=0x7FC0)
+    expected = helpers.expected_output(w)
+    ranges, templates, cu = helpers.fixed_slice_plan(histories, q_lens, tile, 1 << 20)
+    print(f"long interior runs hq={hq} hkv={hkv} d={d} tile={tile}", flush=True)
+    actual = gpu_runner.run_sliced_q(w, ranges, templates, cu, device, kind=sdpa.MAP_Q_TOKENS_AND_HEADS, max_q_tokens=tile,
+                                     max_q_heads=hq // hkv, stage=64, direct=True)
+    helpers.assert_parity(actual, expected, f"long interior runs hq={hq} hkv={hkv}")
+
+
 @pytest.mark.parametrize("hq,hkv,d,tile,fp8", [(64, 8, 128, 32, False), (64, 8, 128, 16, False), (64, 8, 128, 32, True),
                                                (32, 4, 128, 16, True), (32, 8, 128, 4, False), (24, 4, 256, 16, False),
                                                (24, 4, 256, 16, True)])
