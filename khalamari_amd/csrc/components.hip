@@ -47,10 +47,16 @@ static TileKernelChoice select_tile_kernel(uint32_t head_dim, uint32_t coordinat
     // do not follow the largest score.  (One kernel holding both kinds of interior loop spills.)  These are the two-
     // column-tile kernels at D 128 and the eight-wave tile at D 256 (523 -> 638 TFLOP/s on 2048-token chunks at
     // Hq24/Hkv4); the bandwidth-bound verify tiles have nothing to gain.
+    // Twelve waves of one column tile each for 129..192 coordinates at D 256 (32 tokens x 6 Q heads of a KV head: no idle
+    // column, three waves per SIMD); bf16 pages only, FP8 pages keep the 256-column build for such tiles.
+    if (head_dim == 256 && coordinates > 128 && coordinates <= 192 && kv_dtype != KHM_DTYPE_FP8_E4M3FN) {
+        if (direct) return {tile_map_kernel<256, 1, 12, 32, 4, 1, false, true>, 768, (uint32_t)TileSmem<256, 32, 4, 512, true>::kBytes};
+        return {tile_map_kernel<256, 1, 12, 32, 4, 1>, 768, (uint32_t)TileSmem<256, 32, 4, 512, true>::kBytes};
+    }
     if (direct && head_dim == 256 && coordinates > 64 && coordinates <= 128) {
         if (kv_dtype == KHM_DTYPE_FP8_E4M3FN)
             return {tile_map_kernel<256, 1, 8, 32, 4, 1, true, true>, 512, (uint32_t)TileSmem<256, 32, 4>::kBytes};
-        return {tile_map_kernel<256, 1, 8, 32, 4, 1, false, true>, 512, (uint32_t)TileSmem<256, 32, 4>::kBytes};
+        return {tile_map_kernel<256, 1, 8, 32, 4, 1, false, true>, 512, (uint32_t)TileSmem<256, 32, 4, 512, true>::kBytes};
     }
     if (direct && head_dim == 128 && coordinates > 64) {
         const bool wide = coordinates > 128;
@@ -90,9 +96,9 @@ static TileKernelChoice select_tile_kernel(uint32_t head_dim, uint32_t coordinat
         // 65..128 coordinates: eight waves of one column tile each (167 VGPRs, two waves per SIMD) rather than four waves
         // of two (256 VGPRs + 167 AGPRs, one wave per SIMD, nothing to overlap its waits with): 414 -> 527 TFLOP/s on a
         // batch of 2048-token chunks at Hq24/Hkv4.
-        if (coordinates <= 64) return {tile_map_kernel<256, 1, 4, 32, 4, 1>, 256, (uint32_t)TileSmem<256, 32, 4>::kBytes};
-        if (coordinates <= 128) return {tile_map_kernel<256, 1, 8, 32, 4, 1>, 512, (uint32_t)TileSmem<256, 32, 4>::kBytes};
-        return {tile_map_kernel<256, 2, 8, 32, 4, 1>, 512, (uint32_t)TileSmem<256, 32, 4>::kBytes};
+        if (coordinates <= 64) return {tile_map_kernel<256, 1, 4, 32, 4, 1>, 256, (uint32_t)TileSmem<256, 32, 4, 512, true>::kBytes};
+        if (coordinates <= 128) return {tile_map_kernel<256, 1, 8, 32, 4, 1>, 512, (uint32_t)TileSmem<256, 32, 4, 512, true>::kBytes};
+        return {tile_map_kernel<256, 2, 8, 32, 4, 1>, 512, (uint32_t)TileSmem<256, 32, 4, 512, true>::kBytes};
     }
     return {nullptr, 0, 0};
 }

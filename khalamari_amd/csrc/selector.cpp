@@ -284,7 +284,7 @@ static int validate_request_shapes(const khm_selector& selector, const khm_reque
 //       q == 1           -> SlicedKv with all of a KV head's Q heads in one block when ratio <= 8,
 //                           otherwise a one-token sliced-Q tile that still reads K/V once per KV head.
 //       q * ratio <= 64  -> one sliced-Q tile of q tokens x ratio heads (verify blocks).
-//       q >= 16          -> dense prefill: the largest power-of-two token tile with tile * ratio <= 256 (128 at D 256).
+//       q >= 16          -> dense prefill: the largest power-of-two token tile with tile * ratio <= 256 (192 at D 256).
 //       otherwise        -> the largest power-of-two token tile with tile * ratio <= 64.
 //   * KV splits.  A block streams its split once, so splits only need to be short enough to fill the
 //     chip: kTargetBlocks blocks in total and not one more, because the verify kernels hold two (bf16 pages) or four
@@ -308,8 +308,9 @@ static int lookup_variant(const khm_sdpa_config& config, uint32_t queries, khm_s
     }
     // Chunks of 16+ tokens per request are compute-bound: give them the widest tile so each K/V byte staged in
     // LDS feeds as many MFMA columns as possible.  Narrower blocks are bandwidth-bound and stay on small tiles.
-    // At D 256 the 256-column tile does not fit the register file (it spills); 128 columns run a third faster.
-    const uint32_t prefill_columns = config.head_dim > 128 ? kMaxPrefillColumns / 2 : kMaxPrefillColumns;
+    // At D 256 the 256-column tile does not fit the register file (it spills): tiles stop at 192 columns (twelve waves of
+    // one column tile: 32 tokens x 6 heads of a group-6 model) and otherwise at 128.
+    const uint32_t prefill_columns = config.head_dim > 128 ? 3 * kMaxPrefillColumns / 4 : kMaxPrefillColumns;
     const uint32_t max_columns = queries >= 16 ? prefill_columns : kMaxColumns;
     uint32_t heads = std::min(ratio, max_columns);
     uint32_t tile = queries;

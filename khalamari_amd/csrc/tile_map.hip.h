@@ -32,26 +32,28 @@ namespace khm {
 
 // LDS tiles.  A tile is made of units: the 1024 bytes one wave load (64 lanes x 16 bytes) delivers, which the loading
 // lanes may fill with any 64 of the 16-byte chunks of the rows the unit covers.
-// LINEAR (bf16 pages at head dim 128, rows of 256 bytes, four rows per unit): every fragment a lane reads during a slice
-// sits at a fixed distance from the lane's first one, so the reads of a slice share one address register and differ in
-// their immediate offsets only.  A unit holds its rows in pieces of 64 bytes, piece q of row r at 256 q + 64 r, which
-// keeps four neighbouring lanes of a wave load on 64 contiguous bytes of a page; inside a K piece the four chunks are
-// XORed with the unit index, and V units lie 1056 bytes apart, so that the lanes the LDS serves together (sixteen
-// rows of a K read, two units of a transposed V read) fall on different banks.
-// Other tiles keep rows whole and XOR the chunk index with the row (see the swizzles in the kernel).
+// LINEAR (bf16 pages): every fragment a lane reads during a slice sits at a fixed distance from the lane's first one,
+// so the reads of a slice share one address register and differ in their immediate offsets only.  A unit covers 256
+// bytes (128 dims) of four rows - at head dim 256 a row group has two units, one per half of the row - in pieces of 64
+// bytes: piece q of row r at 256 q + 64 r, which keeps four neighbouring lanes of a wave load on 64 contiguous bytes
+// of a page.  What keeps the lanes that the LDS serves in one pass on different banks: a ds_read_b128 is served in
+// four passes of four lane quads each - quads {0,3,5,6}, {1,2,4,7}, {8,11,13,14}, {9,10,12,15} (measured: a layout
+// that is conflict-free for sixteen consecutive lanes only shows one conflict cycle per pass) - so the four chunks of
+// a K piece are permuted by (-chunk ^ row group) & 3; a ds_read_b64_tr_b16 is served in two passes of 32 lanes, which
+// touch two V units, and V units lie 1056 bytes apart so that these fall on different halves of every 64 bytes.
+// Other tiles (FP8 pages) keep rows whole and XOR the chunk index with the row (see the swizzles in the kernel).
 template <int D, int BK, int NSTAGES, int ROW_BYTES = D * 2, bool LINEAR = false>
 struct TileSmem {
-    static_assert(!LINEAR || ROW_BYTES == 256, "the linear layout is written for rows of 256 bytes");
+    static_assert(!LINEAR || ROW_BYTES == 2 * D, "the linear layout is written for bf16 rows");
     static constexpr int kRowBytes = ROW_BYTES;
-    static constexpr int kRowsPerUnit = 1024 / ROW_BYTES;
-    static constexpr int kUnitsPerTile = BK / kRowsPerUnit;
+    static constexpr int kUnitsPerTile = BK * ROW_BYTES / 1024;
     static constexpr int kVUnitPitch = LINEAR ? 1056 : 1024;
-    static constexpr int kKTileBytes = BK * kRowBytes;
+    static constexpr int kKTileBytes = kUnitsPerTile * 1024;
     static constexpr int kVTileBytes = kUnitsPerTile * kVUnitPitch;
     static constexpr int kBytes = NSTAGES * (kKTileBytes + kVTileBytes);
 };
 // which kernels use the linear layout (the host sizes the dynamic LDS with the same rule)
-constexpr bool tile_layout_is_linear(int head_dim, bool fp8_pages) { return head_dim == 128 && !fp8_pages; }
+constexpr bool tile_layout_is_linear(int head_dim, bool fp8_pages) { return (head_dim == 128 || head_dim == 256) && !fp8_pages; }
 
 
 // 16 bytes per lane from global memory to LDS: lane l of the wave reads uniform_base + lane_offset and lands at
@@ -97,22 +99,30 @@ __device__ __forceinline__ void barrier_keeping_loads_in_flight() {
 // DIRECT: the instantiation only ever writes final output (p.output_mode == kMapDirectBf16, which the host guarantees);
 // it exists where following the largest score is worth compiling out, see the untracked slices below.
 template <int D, int NTW, int NWAVES, int BK, int NSTAGES, int MIN_BLOCKS, bool KV8 = false, bool DIRECT = false>
-__global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const MapParams p) {
+__global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) __attribute__((amdgpu_waves_per_eu(NWAVES * MIN_BLOCKS / 4, NWAVES * MIN_BLOCKS / 4)))
+void tile_map_kernel(const MapParams p) {
     constexpr int KS = D / 32;                      // QK k-steps
     constexpr int MT = D / 16;                      // PV dim tiles
     constexpr int SL = BK / 32;                     // slices per tile
     constexpr int PAGE_ROW = D * (KV8 ? 1 : 2);     // bytes of one K/V row in a page
     constexpr int CPR = PAGE_ROW / 16;              // 16-byte chunks per K/V row in a page
-    constexpr int RPL = 64 / CPR;                   // rows per wave load
-    constexpr int UNITS = BK / RPL;                 // wave loads per plane and tile
-    constexpr int UPW = UNITS / NWAVES;             // ... per wave
-    constexpr int LPW = 2 * UPW;                    // K + V loads per wave and tile
-    static_assert(UNITS % NWAVES == 0 && UPW >= 1, "tile loads must divide evenly over the waves");
+    constexpr bool LINEAR = tile_layout_is_linear(D, KV8);
+    constexpr int HALVES = LINEAR ? D / 128 : 1;    // linear layout: wave loads per row group (each takes 128 dims of four rows)
+    constexpr int RPL = LINEAR ? 4 : 64 / CPR;      // rows per wave load
+    constexpr int UNITS = BK * CPR / 64;            // wave loads per plane and tile
+    // PAIRED: the units divide evenly over the waves; a wave then loads K and V of the same units, which share their page
+    // id and scalar base.  Otherwise (twelve waves over sixteen units) the 2 * UNITS loads of a tile are dealt out as one
+    // list, two or three to a wave, and a wave with fewer repeats its last one so that every wave counts the same number
+    // of loads per tile (the waits are compile-time constants).
+    constexpr bool PAIRED = UNITS % NWAVES == 0;
+    constexpr int UPW = PAIRED ? UNITS / NWAVES : 1;                           // units per wave (paired form)
+    constexpr int LPW = PAIRED ? 2 * UPW : (2 * UNITS + NWAVES - 1) / NWAVES;  // loads per wave and tile
+    constexpr int IDS = PAIRED ? UPW : LPW;                                    // page ids per wave and tile
+    static_assert(PAIRED || !KV8, "FP8 tiles are written for evenly divided units");
     static_assert((SL == 1 || SL == 2) && NSTAGES >= 3 && NSTAGES <= 5, "unsupported tiling");
     constexpr bool RAW8 = KV8 && NTW == 1 && NWAVES == 4;   // raw FP8 codes in LDS, decoded by the waves that read them
     constexpr bool STAGED8 = KV8 && !RAW8;       // FP8 tiles decoded once on their way into bf16 LDS tiles
     static_assert(!STAGED8 || NSTAGES == 4, "the register-staged FP8 path is written for a ring of four tiles");
-    constexpr bool LINEAR = tile_layout_is_linear(D, KV8);
     using Smem = TileSmem<D, BK, NSTAGES, RAW8 ? D : 2 * D, LINEAR>;
     constexpr int ROW = Smem::kRowBytes;
     constexpr int V_UNIT = Smem::kVUnitPitch;
@@ -122,22 +132,25 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     auto k_swizzle_of = [](uint32_t row) -> uint32_t { return (RAW8 && D == 128) ? ((row >> 1) & 7u) : (row & 15u); };
     auto v_swizzle_of = [](uint32_t row) -> uint32_t { return RAW8 ? (D == 128 ? ((row >> 1) & 7u) : (row & 15u)) : ((row & 7u) << 1); };
     // Where chunk `chunk` (16 bytes) of tile row `row` sits inside its K or V tile in LDS.
+    // Unit n of a tile (the n-th wave load of a plane): its first row, and its place among the tile's units in LDS.
+    auto unit_first_row = [](uint32_t n) -> uint32_t { return (n / HALVES) * RPL; };
+    auto unit_position = [](uint32_t n) -> uint32_t { return LINEAR ? (n % HALVES) * (BK / 4) + n / HALVES : n; };
     auto k_place = [&](uint32_t row, uint32_t chunk) -> uint32_t {
-        if constexpr (LINEAR) return (row >> 2) * 1024 + (chunk >> 2) * 256 + ((row & 3u) << 6) + ((((0u - chunk) ^ (row >> 2)) & 3u) << 4);
+        if constexpr (LINEAR) return ((chunk >> 4) * (BK / 4) + (row >> 2)) * 1024 + ((chunk >> 2) & 3u) * 256 + ((row & 3u) << 6) + ((((0u - chunk) ^ (row >> 2)) & 3u) << 4);
         else return row * ROW + ((chunk ^ k_swizzle_of(row)) << 4);
     };
     auto v_place = [&](uint32_t row, uint32_t chunk) -> uint32_t {
-        if constexpr (LINEAR) return (row >> 2) * V_UNIT + (chunk >> 2) * 256 + ((row & 3u) << 6) + ((chunk & 3u) << 4);
+        if constexpr (LINEAR) return ((chunk >> 4) * (BK / 4) + (row >> 2)) * V_UNIT + ((chunk >> 2) & 3u) * 256 + ((row & 3u) << 6) + ((chunk & 3u) << 4);
         else return row * ROW + ((chunk ^ v_swizzle_of(row)) << 4);
     };
     // The inverse, for the lane that fills 16-byte slot `slot` of unit `unit` of a tile: row inside the tile and chunk.
     struct Source { uint32_t row, chunk; };
     auto k_source_of = [&](uint32_t unit, uint32_t slot) -> Source {
-        if constexpr (LINEAR) return Source{unit * 4 + ((slot >> 2) & 3u), (slot >> 4) * 4 + ((0u - (slot ^ unit)) & 3u)};
+        if constexpr (LINEAR) return Source{unit_first_row(unit) + ((slot >> 2) & 3u), (unit % HALVES) * 16 + (slot >> 4) * 4 + ((0u - (slot ^ (unit / HALVES))) & 3u)};
         else { const uint32_t row = unit * RPL + slot / CPR; return Source{row, (slot % CPR) ^ k_swizzle_of(row)}; }
     };
     auto v_source_of = [&](uint32_t unit, uint32_t slot) -> Source {
-        if constexpr (LINEAR) return Source{unit * 4 + ((slot >> 2) & 3u), (slot >> 4) * 4 + (slot & 3u)};
+        if constexpr (LINEAR) return Source{unit_first_row(unit) + ((slot >> 2) & 3u), (unit % HALVES) * 16 + (slot >> 4) * 4 + (slot & 3u)};
         else { const uint32_t row = unit * RPL + slot / CPR; return Source{row, (slot % CPR) ^ v_swizzle_of(row)}; }
     };
 
@@ -326,13 +339,27 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     // tile is issued, and the load address is a scalar base plus a 32-bit lane offset.
     // Rows outside [blk_lo, blk_hi) may hold anything (unused page slots): their loads are redirected to the nearest
     // visible token, so LDS only ever holds finite K/V and a zero weight really contributes zero.
-    typedef uint32_t TileIds __attribute__((ext_vector_type(UPW < 2 ? 2 : UPW)));
+    // Load j of this wave: which unit of the tile, K or V plane, and which of the wave's page ids it uses (all wave-uniform).
+    const uint32_t first_load = PAIRED ? 0u : (uint32_t)(wave * 2 * UNITS) / NWAVES;
+    const uint32_t num_loads = PAIRED ? (uint32_t)LPW : (uint32_t)((wave + 1) * 2 * UNITS) / NWAVES - first_load;
+    auto load_index = [&](int j) -> uint32_t { return first_load + ((uint32_t)j < num_loads ? (uint32_t)j : num_loads - 1); };
+    auto load_unit = [&](int j) -> uint32_t { return PAIRED ? (uint32_t)(wave * UPW + j / 2) : load_index(j) % UNITS; };
+    auto load_is_v = [&](int j) -> bool { return PAIRED ? (j & 1) != 0 : load_index(j) >= (uint32_t)UNITS; };
+    auto load_id = [](int j) -> int { return PAIRED ? j / 2 : j; };
+    auto id_unit = [&](int i) -> uint32_t { return PAIRED ? (uint32_t)(wave * UPW + i) : load_unit(i); };
+    auto load_lds_address = [&](int j, uint32_t stage) -> uint32_t {
+        const uint32_t position = unit_position(load_unit(j));
+        return load_is_v(j) ? v_lds_address + stage * Smem::kVTileBytes + position * V_UNIT : k_lds_address + stage * Smem::kKTileBytes + position * 1024;
+    };
+    auto load_source = [&](int j) -> Source { return load_is_v(j) ? v_source_of(load_unit(j), lane) : k_source_of(load_unit(j), lane); };
+
+    typedef uint32_t TileIds __attribute__((ext_vector_type(IDS < 2 ? 2 : IDS)));
     auto fetch_ids = [&](uint32_t tile) __attribute__((always_inline)) -> TileIds {
         TileIds ids;
         const uint32_t last_page = p.pages_per_request_layer - 1;
 #pragma unroll
-        for (int i = 0; i < UPW; ++i) {
-            uint32_t token = first_token + tile * BK + (wave * UPW + i) * RPL;
+        for (int i = 0; i < IDS; ++i) {
+            uint32_t token = first_token + tile * BK + unit_first_row(id_unit(i));
             token = token < blk_lo ? blk_lo : token;
             token = token >= blk_hi ? blk_hi - 1 : token;
             const uint32_t page = token >> tpp_shift;
@@ -341,42 +368,34 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         return ids;
     };
     // Lane offsets of a wave load inside its page.  A tile that lies wholly inside [blk_lo, blk_hi) needs no clamp and,
-    // BK being a multiple of the page size, its offsets do not depend on the tile: those live in registers.
-    uint32_t k_lane_offset[UPW], v_lane_offset[UPW];
+    // BK being a multiple of the page size, its offsets do not depend on the tile: those live in registers.  All loads
+    // use one scalar base (the K plane of their page); the offsets of V loads carry the distance to the V plane.
+    const uint32_t v_plane_distance = (uint32_t)(plane_v - plane_k);
+    uint32_t lane_offset[LPW];
 #pragma unroll
-    for (int i = 0; i < UPW; ++i) {
-        const Source k_source = k_source_of(wave * UPW + i, lane), v_source = v_source_of(wave * UPW + i, lane);
-        k_lane_offset[i] = ((first_token + k_source.row) & (tpp - 1)) * PAGE_ROW + (k_source.chunk << 4);
-        // K and V of a wave load share one scalar base (the K plane of their page): the V offsets carry the distance
-        v_lane_offset[i] = ((first_token + v_source.row) & (tpp - 1)) * PAGE_ROW + (v_source.chunk << 4) + (uint32_t)(plane_v - plane_k);
+    for (int j = 0; j < LPW; ++j) {
+        const Source source = load_source(j);
+        lane_offset[j] = ((first_token + source.row) & (tpp - 1)) * PAGE_ROW + (source.chunk << 4) + (load_is_v(j) ? v_plane_distance : 0u);
     }
+    const unsigned char* const k_plane_base = p.kv_pages + plane_k;
     auto issue_tile = [&](uint32_t tile, const TileIds ids) __attribute__((always_inline)) {
         const uint32_t stage = tile % NSTAGES;
         const uint32_t tile_token = first_token + tile * BK;
         if (tile_token >= blk_lo && tile_token + BK <= blk_hi) {
 #pragma unroll
-            for (int i = 0; i < UPW; ++i) {
-                const uint32_t unit = wave * UPW + i;                                  // wave-uniform
-                const unsigned char* page = p.kv_pages + plane_k + (uint64_t)ids[i] * p.page_bytes;   // scalar
-                load_to_lds_b128(page, k_lane_offset[i], k_lds_address + stage * Smem::kKTileBytes + unit * 1024);
-                load_to_lds_b128(page, v_lane_offset[i], v_lds_address + stage * Smem::kVTileBytes + unit * V_UNIT);
-            }
+            for (int j = 0; j < LPW; ++j)
+                load_to_lds_b128(k_plane_base + (uint64_t)ids[load_id(j)] * p.page_bytes, lane_offset[j], load_lds_address(j, stage));
             return;
         }
         // first or last tile of the range: rows outside it are redirected, which changes their offsets
 #pragma unroll
-        for (int i = 0; i < UPW; ++i) {
-            const uint32_t unit = wave * UPW + i;
-            const Source k_source = k_source_of(unit, lane), v_source = v_source_of(unit, lane);
-            auto in_page_of = [&](uint32_t row) {
-                uint32_t token = tile_token + row;
-                token = token < blk_lo ? blk_lo : token;
-                token = token >= blk_hi ? blk_hi - 1 : token;
-                return (token & (tpp - 1)) * PAGE_ROW;
-            };
-            const unsigned char* page = p.kv_pages + (uint64_t)ids[i] * p.page_bytes;
-            load_to_lds_b128(page + plane_k, in_page_of(k_source.row) + (k_source.chunk << 4), k_lds_address + stage * Smem::kKTileBytes + unit * 1024);
-            load_to_lds_b128(page + plane_v, in_page_of(v_source.row) + (v_source.chunk << 4), v_lds_address + stage * Smem::kVTileBytes + unit * V_UNIT);
+        for (int j = 0; j < LPW; ++j) {
+            const Source source = load_source(j);
+            uint32_t token = tile_token + source.row;
+            token = token < blk_lo ? blk_lo : token;
+            token = token >= blk_hi ? blk_hi - 1 : token;
+            const uint32_t offset = (token & (tpp - 1)) * PAGE_ROW + (source.chunk << 4) + (load_is_v(j) ? v_plane_distance : 0u);
+            load_to_lds_b128(k_plane_base + (uint64_t)ids[load_id(j)] * p.page_bytes, offset, load_lds_address(j, stage));
         }
     };
 
@@ -386,21 +405,16 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         TileIds ids;
         const uint32_t last_page = p.pages_per_request_layer - 1;
 #pragma unroll
-        for (int i = 0; i < UPW; ++i) {
-            const uint32_t page = (first_token + tile * BK + (wave * UPW + i) * RPL) >> tpp_shift;
+        for (int i = 0; i < IDS; ++i) {
+            const uint32_t page = (first_token + tile * BK + unit_first_row(id_unit(i))) >> tpp_shift;
             ids[i] = load_uniform_u32(table, page < last_page ? page : last_page);   // the tile after the last one requested is read, not used
         }
         return ids;
     };
-    const unsigned char* const k_plane_base = p.kv_pages + plane_k;
     auto issue_interior_tile = [&](uint32_t stage, const TileIds ids) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < UPW; ++i) {
-            const uint32_t unit = wave * UPW + i;
-            const unsigned char* page = k_plane_base + (uint64_t)ids[i] * p.page_bytes;
-            load_to_lds_b128(page, k_lane_offset[i], k_lds_address + stage * Smem::kKTileBytes + unit * 1024);
-            load_to_lds_b128(page, v_lane_offset[i], v_lds_address + stage * Smem::kVTileBytes + unit * V_UNIT);
-        }
+        for (int j = 0; j < LPW; ++j)
+            load_to_lds_b128(k_plane_base + (uint64_t)ids[load_id(j)] * p.page_bytes, lane_offset[j], load_lds_address(j, stage));
     };
 
     // FP8 pages: one tile in registers, decoded into the bf16 LDS layout the direct loads would have produced
@@ -457,7 +471,10 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
     const uint32_t v_row = RAW8 ? ((r16 >> 1) < 4 ? g * 4 + (r16 >> 1) : 16 + g * 4 + (r16 >> 1) - 4) : g * 4 + (r16 >> 2);
     const uint32_t v_swizzle = RAW8 ? v_swizzle_of(v_row) : ((r16 & 3) >> 1) ^ ((v_row & 7) << 1);
     const uint32_t v_base = LINEAR ? v_place(v_row, (r16 & 3) >> 1) + (r16 & 1) * 8 : v_row * ROW + (r16 & 1) * 8;
-    constexpr uint32_t kSixteenRows = LINEAR ? 4 * V_UNIT : 16 * ROW;   // V rows 16 apart in a tile
+    constexpr uint32_t kKSliceBytes = LINEAR ? 8 * 1024 : 32 * ROW;      // from a 32-token slice of a tile to the next
+    constexpr uint32_t kVSliceBytes = LINEAR ? 8 * V_UNIT : 32 * ROW;
+    constexpr uint32_t kSixteenRows = LINEAR ? 4 * V_UNIT : 16 * ROW;    // V rows 16 apart in a tile
+    constexpr uint32_t kSixteenKRows = LINEAR ? 4 * 1024 : 16 * ROW;     // K rows 16 apart in a tile
     auto v_fragment = [&](const unsigned char* v_src, int mt) __attribute__((always_inline)) -> bf16x8 {
         if constexpr (RAW8) {
             typedef int CodeWords __attribute__((ext_vector_type(2)));
@@ -465,7 +482,7 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             const CodeWords codes = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CodeWords __attribute__((address_space(3)))*)(address));
             return __builtin_bit_cast(bf16x8, fp8x8_to_bf16x8(make_uint2((uint32_t)codes[0], (uint32_t)codes[1])));
         } else {
-            const unsigned char* address = v_src + v_base + (LINEAR ? (uint32_t)((mt >> 1) * 256 + (mt & 1) * 32) : ((mt * 2) ^ v_swizzle) << 4);
+            const unsigned char* address = v_src + v_base + (LINEAR ? (uint32_t)((mt >> 3) * (BK / 4) * V_UNIT + ((mt & 7) >> 1) * 256 + (mt & 1) * 32) : ((mt * 2) ^ v_swizzle) << 4);
             const uint2 lo = __builtin_bit_cast(uint2, lds_read_tr16(address));
             const uint2 hi = __builtin_bit_cast(uint2, lds_read_tr16(address + kSixteenRows));
             return __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
@@ -512,9 +529,9 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             for (int rt = 0; rt < 2; ++rt) {
                 bf16x8 a;
                 if constexpr (RAW8) {
-                    a = __builtin_bit_cast(bf16x8, fp8x8_to_bf16x8(*reinterpret_cast<const uint2*>(k_src + k_offset[ks] + rt * 16 * ROW)));
+                    a = __builtin_bit_cast(bf16x8, fp8x8_to_bf16x8(*reinterpret_cast<const uint2*>(k_src + k_offset[ks] + rt * kSixteenKRows)));
                 } else {
-                    a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(k_src + k_offset[ks] + rt * 16 * ROW));
+                    a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(k_src + k_offset[ks] + rt * kSixteenKRows));
                 }
 #pragma unroll
                 for (int nt = 0; nt < NTW; ++nt)
@@ -699,10 +716,10 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
         else wait_vmem_outstanding<0>();
     };
     auto k_slice = [&](uint32_t slice) __attribute__((always_inline)) -> const unsigned char* {
-        return k_lds + ((slice / SL) % NSTAGES) * Smem::kKTileBytes + (slice % SL) * 32 * ROW;
+        return k_lds + ((slice / SL) % NSTAGES) * Smem::kKTileBytes + (slice % SL) * kKSliceBytes;
     };
     auto v_slice = [&](uint32_t slice) __attribute__((always_inline)) -> const unsigned char* {
-        return v_lds + ((slice / SL) % NSTAGES) * Smem::kVTileBytes + (slice % SL) * (Smem::kVTileBytes / SL);
+        return v_lds + ((slice / SL) % NSTAGES) * Smem::kVTileBytes + (slice % SL) * kVSliceBytes;
     };
     Scores pending;
     TileIds upcoming = fetch_ids(NSTAGES - 1);
@@ -758,7 +775,7 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
             }
         }
     };
-    // Steady state of an interior run (direct loads, two slices per tile, untracked weights): every tile of
+    // Steady state of an interior run (direct loads, untracked weights): every tile of
     // [tile_begin, tile_end) has its successor's first slice in the range, and the tile NSTAGES - 1 ahead exists and lies
     // wholly inside the block's KV range.  One straight-line body per tile: a fixed wait, the barrier, unconditional
     // requests; the compiler is free to mix the S^T of the next slice with the softmax of this one.
@@ -777,8 +794,13 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
                 ahead = fetch_ids_interior(tile + NSTAGES);
             };
             auto nothing = []() __attribute__((always_inline)) {};
-            process_slice(no, no, untracked_anchored, 0u, pending, k_tile, k_tile + 32 * ROW, v_tile, request_next);
-            process_slice(no, no, untracked_anchored, 0u, pending, k_tile + 32 * ROW, k_lds + next_stage * Smem::kKTileBytes, v_tile + Smem::kVTileBytes / 2, nothing);
+            const unsigned char* k_following = k_lds + next_stage * Smem::kKTileBytes;
+            if constexpr (SL == 2) {
+                process_slice(no, no, untracked_anchored, 0u, pending, k_tile, k_tile + kKSliceBytes, v_tile, request_next);
+                process_slice(no, no, untracked_anchored, 0u, pending, k_tile + kKSliceBytes, k_following, v_tile + kVSliceBytes, nothing);
+            } else {
+                process_slice(no, no, untracked_anchored, 0u, pending, k_tile, k_following, v_tile, request_next);
+            }
         }
     };
 
@@ -843,7 +865,7 @@ __global__ __launch_bounds__(NWAVES * 64, MIN_BLOCKS) void tile_map_kernel(const
 #pragma unroll
                 for (int nt = 0; nt < NTW; ++nt) unanchored = unanchored | (lane_top[nt] == -INFINITY);
                 uint32_t steady_end = head_end;
-                if constexpr (!STAGED8 && SL == 2) {
+                if constexpr (!STAGED8) {
                     // tiles t with t + NSTAGES - 1 a whole tile inside [blk_lo, blk_hi): (t + NSTAGES) * BK <= blk_hi - first_token
                     const uint32_t whole_tiles = (blk_hi - first_token) / BK;
                     uint32_t limit = whole_tiles >= (uint32_t)NSTAGES ? whole_tiles - (NSTAGES - 1) : 0;

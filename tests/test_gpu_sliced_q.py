@@ -359,7 +359,8 @@ def test_selector_and_metadata_drive_the_kernels_end_to_end(device):
         assert np.all(out[w.num_tokens:].cpu().numpy() == POISON)
 
 
-@pytest.mark.parametrize("hq,hkv,d,tile", [(64, 8, 128, 32), (32, 4, 128, 16), (24, 4, 256, 16), (16, 2, 256, 32)])
+@pytest.mark.parametrize("hq,hkv,d,tile", [(64, 8, 128, 32), (32, 4, 128, 16), (24, 4, 256, 16), (16, 2, 256, 32), (24, 4, 256, 32),
+                                           (12, 2, 256, 32)])
 def test_chunked_prefill_onto_a_paged_prefix(device, hq, hkv, d, tile):
     """Config-5 shape at reduced size: causal chunks appended to paged prefixes (including an empty prefix), wide
     Q tiles on the LDS-shared K/V kernel, direct output and split-KV + Reduce."""
@@ -377,7 +378,7 @@ def test_chunked_prefill_onto_a_paged_prefix(device, hq, hkv, d, tile):
         helpers.assert_parity(actual, expected, f"prefill tile={tile} slice={kv_slice} direct={direct}")
 
 
-@pytest.mark.parametrize("hq,hkv,d,tile", [(16, 2, 128, 32), (8, 2, 128, 32)])
+@pytest.mark.parametrize("hq,hkv,d,tile", [(16, 2, 128, 32), (8, 2, 128, 32), (12, 2, 256, 32), (12, 2, 256, 16)])
 def test_long_interior_runs_of_a_prefill_tile_checked_on_every_row(device, hq, hkv, d, tile):
     """Prefixes of several thousand keys, so that nearly all tiles of a block are interior ones that run in the
     steady-state loop of the direct-output builds (unconditional requests, weights that do not follow the largest
@@ -396,7 +397,7 @@ def test_long_interior_runs_of_a_prefill_tile_checked_on_every_row(device, hq, h
 
 @pytest.mark.parametrize("hq,hkv,d,tile,fp8", [(64, 8, 128, 32, False), (64, 8, 128, 16, False), (64, 8, 128, 32, True),
                                                (32, 4, 128, 16, True), (32, 8, 128, 4, False), (24, 4, 256, 16, False),
-                                               (24, 4, 256, 16, True)])
+                                               (24, 4, 256, 16, True), (24, 4, 256, 32, False)])
 def test_scores_that_keep_outgrowing_the_running_reference(device, hq, hkv, d, tile, fp8):
     """Every score of a sequence rises steadily along the context (by some 60 octaves over 3000 keys), so later scores
     exceed the earlier maximum by far more than any rescaling threshold, over and over: the reference-moving path of
