@@ -14,6 +14,8 @@ import bench
 from khalamari_amd import sdpa, sliced_q
 from khalamari_amd._lib import DTYPE_BF16, DTYPE_F32, ReplayU32
 
+from oracle import gqa_oracle as oracle
+
 from . import gpu_runner, helpers
 from .test_gpu_full_size import _oracle_rows, _sampled_tokens
 
@@ -97,3 +99,42 @@ def test_tile_arithmetic_meets_the_strict_gate(device, index):
     stats = helpers.assert_strict_parity(actual, expected, f"config {index}, f32 before the output cast")
     print(stats)
     helpers.record_parity(f"config{index} full size, f32 before the output cast, unsplit, {len(tokens)} tokens", stats)
+
+
+@pytest.mark.parametrize("index,partial", [(2, "f32"), (2, "bf16"), (3, "f32"), (3, "bf16")])
+def test_split_decode_meets_the_strict_gate(device, monkeypatch, index, partial):
+    """Configs 2 and 3 with the partitions BASELINE gives them (512 / 2048 tokens): the Map's partial states and statistics
+    are read back and merged on the host by the oracle's Reduce, so the result is an f32 value that has been through the
+    split path but not through the bf16 output cast, and is held to the strict gate against the unsplit oracle
+    (sliced_kv_test.rs:511-532 compares the split path with the reference the same way).  With f32 partial states this
+    isolates the arithmetic of Map + log-sum-exp merge; with the default bf16 partial states the partial format's own
+    rounding (2^-9 of each partial) is in the figure, which is recorded beside the first and held to the combined bound."""
+    from khalamari_amd import batch_metadata
+
+    monkeypatch.setenv("KHM_BENCH_PARTIAL", partial)
+    monkeypatch.setenv("KHM_BENCH_FUSED", "0")
+    workload = bench.Workload(index, device, num_pools=1)
+    spec = workload.spec
+    hq, d = spec["hq"], spec["d"]
+    templates = workload.replay_shape.num_sdpa_map_task_templates
+    assert templates > workload.num_tokens            # the KV ranges really are split
+    workload.launch_map(workload.kv_pools[0])
+    torch.cuda.synchronize()
+    scratch = workload._keep[1]
+    sums = scratch.partial_exp_sums.view(torch.float32).cpu().numpy()[:templates * hq]
+    maxs = scratch.partial_max_logits.view(torch.float32).cpu().numpy()[:templates * hq]
+    if partial == "f32":
+        states = scratch.partial_output.view(torch.float32).cpu().numpy()[:templates * hq * d]
+    else:
+        states = gpu_runner.bf16_tensor_to_f32(scratch.partial_output.view(torch.int16)).reshape(-1)[:templates * hq * d]
+    cu = workload.metadata.host(batch_metadata.CU_SDPA_PARTIAL_OUTPUTS)[:workload.num_tokens + 1]
+    actual = oracle.reduce_sliced_kv(sums, maxs, states, cu, workload.num_tokens, hq, d)
+    tokens = list(range(workload.num_tokens))
+    expected = _oracle_rows(workload, workload.kv_pools[0], tokens)
+    name = f"config{index} full size, {spec['kv_slice']}-token partitions, {partial} partial states merged in f32 on the host, before the output cast"
+    if partial == "f32":
+        stats = helpers.assert_strict_parity(actual, expected, name)
+    else:
+        stats = helpers.assert_parity(actual, expected, name)
+    print(stats)
+    helpers.record_parity(f"{name}, {len(tokens)} tokens", stats)
