@@ -52,7 +52,6 @@ CONFIGS[EXTRA_PREFILL_D256] = dict(name="extra: B=8 chunked prefill, 2048-token 
 
 
 SLAB_BYTES = 4096
-CLOCK_PROBE = True   # --no-clock-probe: counter runs want the Map launches alone on the device
 _slab_reader_lib = None
 
 
@@ -87,63 +86,7 @@ def _bench_aid_lib():
         _slab_reader_lib.bench_slab_read.restype = ctypes.c_int
         _slab_reader_lib.bench_slab_read.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint32,
                                                      ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
-        _slab_reader_lib.bench_mfma_sustained_operand_bytes.restype = ctypes.c_uint64
-        _slab_reader_lib.bench_mfma_sustained_sink_bytes.restype = ctypes.c_uint64
-        _slab_reader_lib.bench_mfma_sustained_sink_bytes.argtypes = [ctypes.c_uint32]
-        _slab_reader_lib.bench_mfma_sustained_flops.restype = ctypes.c_double
-        _slab_reader_lib.bench_mfma_sustained_flops.argtypes = [ctypes.c_uint32, ctypes.c_uint32]
-        _slab_reader_lib.bench_clock_probe.restype = ctypes.c_int
-        _slab_reader_lib.bench_clock_probe.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_void_p]
-        _slab_reader_lib.bench_mfma_sustained.restype = ctypes.c_int
-        _slab_reader_lib.bench_mfma_sustained.argtypes = [ctypes.c_uint32, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_uint64,
-                                                          ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p]
     return _slab_reader_lib
-
-
-def mfma_sustained_table(device, steps: int = 400000) -> list:
-    """Rate and shader clock of a loop of bare bf16 MFMA instructions (`bench_mfma_sustained.hip`, eight waves per CU, no
-    memory traffic) for both tile shapes, on operands that are all 1.0 and on operands drawn from N(0, 1).  The first
-    shows the published peak; the second is what the chip sustains on data like attention's, where the clock governor
-    settles below the 2.4 GHz the published figure assumes: the ceiling any kernel on real data runs under."""
-    import ctypes
-
-    import torch
-
-    lib = _bench_aid_lib()
-    compute_units = torch.cuda.get_device_properties(device).multi_processor_count
-    operand_bytes = int(lib.bench_mfma_sustained_operand_bytes())
-    sink = torch.empty(int(lib.bench_mfma_sustained_sink_bytes(compute_units)) // 4, dtype=torch.float32, device=device)
-    counters = torch.zeros(2, dtype=torch.int64, device=device)
-    generator = torch.Generator(device="cpu")
-    generator.manual_seed(7)
-    rows = []
-    for tile32 in (0, 1):
-        for operands_name in ("all 1.0", "N(0, 1)"):
-            if operands_name == "all 1.0":
-                host = torch.ones(operand_bytes // 2, dtype=torch.float32)
-            else:
-                host = torch.randn(operand_bytes // 2, generator=generator, dtype=torch.float32)
-            operands = host.to(torch.bfloat16).to(device)
-            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-
-            def launch(count):
-                status = lib.bench_mfma_sustained(tile32, operands.data_ptr(), operand_bytes, sink.data_ptr(), sink.numel() * 4,
-                                                  counters.data_ptr(), 16, compute_units, count, stream)
-                if status != 0:
-                    raise RuntimeError(f"bench_mfma_sustained failed with status {status}")
-
-            launch(steps // 10)
-            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            begin.record()
-            launch(steps)
-            end.record()
-            torch.cuda.synchronize()
-            clock_ticks, real_ticks = (int(v) for v in counters.cpu())
-            seconds = begin.elapsed_time(end) * 1e-3
-            rows.append({"instruction": "v_mfma_f32_32x32x16_bf16" if tile32 else "v_mfma_f32_16x16x32_bf16", "operands": operands_name,
-                         "tflops": lib.bench_mfma_sustained_flops(compute_units, steps) / seconds / 1e12,
-                         "shader_clock_ghz": 0.1 * clock_ticks / max(real_ticks, 1), "ms": seconds * 1e3})
-    return rows
 
 
 def config_key(index: int) -> str:
@@ -427,31 +370,6 @@ class Workload:
                     what="read-only launch of the workload's K/V bytes as random 4 KB slabs of the same pools, evenly split over a resident grid")
         return best
 
-    def shader_clock_during_map(self, map_ms: float) -> float:
-        """GHz of the shader clock while the Map kernel runs: a one-wave kernel on a second stream (`bench_clock_probe`)
-        compares the shader clock counter with the constant 100 MHz counter over a window that lies inside a row of
-        back-to-back Map launches.  It reads the XCD it lands on; runs differ by about 0.1 GHz."""
-        import ctypes
-
-        import torch
-
-        lib = _bench_aid_lib()
-        counters = torch.zeros(2, dtype=torch.int64, device=self.kv_pools[0].device)
-        side = torch.cuda.Stream()
-        ticks_per_ms = 100000
-        launches = max(6, int(12.0 / max(map_ms, 1e-3)))
-        window_ms = min(0.5 * launches * map_ms, 20.0)
-        torch.cuda.synchronize()
-        for i in range(launches):
-            self.launch_map(self.kv_pools[i % len(self.kv_pools)])
-        status = lib.bench_clock_probe(counters.data_ptr(), 16, int(0.25 * launches * map_ms * ticks_per_ms), int(window_ms * ticks_per_ms),
-                                       ctypes.c_void_p(side.cuda_stream))
-        if status != 0:
-            raise RuntimeError(f"bench_clock_probe failed with status {status}")
-        torch.cuda.synchronize()
-        clock_ticks, real_ticks = (int(v) for v in counters.cpu())
-        return 0.1 * clock_ticks / max(real_ticks, 1)
-
     def report(self, steps: int, warmup: int) -> dict:
         ms, map_ms, map_ms_median = self.time_steps(steps, warmup)
         spec = self.spec
@@ -473,12 +391,6 @@ class Workload:
             result.update(bound="mfma", algorithmic_flops=flops, tflops=flops / (ms * 1e-3) / 1e12,
                           map_tflops=flops / (map_ms * 1e-3) / 1e12)
             result["roofline_frac"] = result["map_tflops"] / MFMA_BF16_PEAK_TFLOPS
-            # the published peak is 256 CUs x 4 SIMDs x 1024 flop/clk at 2.4 GHz; the chip runs this kernel at a lower clock
-            if CLOCK_PROBE:
-                clock_ghz = self.shader_clock_during_map(map_ms)
-                result["shader_clock_ghz"] = clock_ghz
-                result["mfma_peak_at_shader_clock_tflops"] = MFMA_BF16_PEAK_TFLOPS * clock_ghz / 2.4
-                result["frac_of_peak_at_shader_clock"] = result["map_tflops"] / result["mfma_peak_at_shader_clock_tflops"]
         else:
             nbytes = self.algorithmic_bytes()
             result.update(bound="hbm", algorithmic_bytes=nbytes, gbps=nbytes / (ms * 1e-3) / 1e9,
@@ -675,10 +587,7 @@ def main() -> int:
                         help="headline config on FP8 E4M3FN pages, the reference's cache format (profiling runs; the default headline keeps bf16 pages)")
     parser.add_argument("--slab-runs", action="store_true",
                         help="time only the read-only launch of the headline config's K/V bytes as contiguous runs of 4 .. 64 KB and print the table as JSON")
-    parser.add_argument("--mfma-sustained", action="store_true",
-                        help="time only the loop of bare bf16 MFMA instructions (rate and shader clock on constant and on random operands) and print the table as JSON")
-    parser.add_argument("--no-clock-probe", action="store_true",
-                        help="prefill configs: skip the one-wave shader clock probe that runs beside extra Map launches (profiling runs)")
+    parser.add_argument("--no-clock-probe", action="store_true", help="accepted and ignored (older command lines)")
     parser.add_argument("--calibration-copy", action="store_true",
                         help="also launch a plain 1 GiB copy kernel, the known-size reference for FETCH_SIZE / WRITE_SIZE counter runs")
     args = parser.parse_args()
@@ -692,9 +601,6 @@ def main() -> int:
         print("bench.py needs an MI355X (no GPU visible)", file=sys.stderr)
         return 2
     device = torch.device("cuda:0")
-    if args.no_clock_probe:
-        global CLOCK_PROBE
-        CLOCK_PROBE = False
     if args.calibration_copy:
         calibration_copy(device)
     if args.producers:
@@ -702,9 +608,6 @@ def main() -> int:
         return 0
     if args.slab_runs:
         print(json.dumps({"slab_runs": slab_run_table(device, args.config)}))
-        return 0
-    if args.mfma_sustained:
-        print(json.dumps({"mfma_sustained": mfma_sustained_table(device)}))
         return 0
     headline = Workload(args.config, device, fp8_pages=args.fp8_pages)
     head = headline.report(args.steps, args.warmup)
@@ -735,10 +638,6 @@ def main() -> int:
             others["producers"] = producer_rows(device)
         except Exception as error:
             others["producers"] = {"error": str(error)}
-        try:
-            others["mfma_sustained"] = mfma_sustained_table(device)
-        except Exception as error:
-            others["mfma_sustained"] = {"error": str(error)}
     prefill = head["bound"] == "mfma"
     line = {
         "metric": "paged GQA prefill bf16 MFMA TFLOP/s" if prefill else "paged GQA decode achieved HBM GB/s (split-KV Map + LSE Reduce per step)",
@@ -768,8 +667,6 @@ def main() -> int:
             "algorithmic_bytes": head.get("algorithmic_bytes"),
             "algorithmic_flops": head.get("algorithmic_flops"),
             "slab_reader": head.get("slab_reader"),
-            "shader_clock_ghz": head.get("shader_clock_ghz"),
-            "frac_of_peak_at_shader_clock": head.get("frac_of_peak_at_shader_clock"),
         },
         "configs": others,
     }

@@ -42,11 +42,10 @@ HIPCC_FLAGS = [
 
 
 def build_bench_aid(verbose: bool = False) -> str:
-    """The kernels bench.py times beside the Map kernels (a read-only slab reader; a loop of bare MFMA instructions that
-    shows the rate and clock the matrix cores sustain): a library of its own at the repository root, not part of
-    `libkhm_gqa_sdpa.so`."""
+    """The read-only slab reader bench.py times beside the bandwidth-bound Map kernels: a library of its own at the
+    repository root, not part of `libkhm_gqa_sdpa.so`."""
     root = os.path.dirname(PACKAGE_DIR)
-    sources = [os.path.join(root, "bench_slab_read.hip"), os.path.join(root, "bench_mfma_sustained.hip")]
+    sources = [os.path.join(root, "bench_slab_read.hip")]
     output = os.path.join(root, "libbench_slab_read.so")
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     command = [hipcc, *HIPCC_FLAGS, "-x", "hip", *sources, "-o", output]

@@ -33,17 +33,4 @@ def test_bench_aid_library_exports_its_entry_points():
     if not os.path.exists(path):
         pytest.skip("libbench_slab_read.so is not built")
     lib = ctypes.CDLL(path)
-    for name in ("bench_slab_read", "bench_mfma_sustained", "bench_mfma_sustained_operand_bytes", "bench_mfma_sustained_sink_bytes",
-                 "bench_mfma_sustained_flops", "bench_clock_probe"):
-        assert hasattr(lib, name), name
-
-
-@pytest.mark.gpu
-def test_gpu_mfma_loop_reaches_a_plausible_rate_and_clock(device):
-    print("bench mfma sustained: 20000 steps per launch", flush=True)
-    rows = bench.mfma_sustained_table(device, steps=20000)
-    assert len(rows) == 4
-    for row in rows:
-        print(row, flush=True)
-        assert 500.0 < row["tflops"] < 2600.0            # 2.5 PFLOP/s is the published dense bf16 peak
-        assert 0.8 < row["shader_clock_ghz"] < 2.6       # 2.4 GHz is the top shader clock
+    assert hasattr(lib, "bench_slab_read")
