@@ -462,8 +462,9 @@ def cpu_baseline(index: int = 2, seconds_hint: float = 20.0) -> dict:
 
 
 def producer_rows(device, steps: int = 20) -> dict:
-    """The two kernels that feed the SDPA, at config 5's prefill shape (8 x 2048 new tokens, Hq=32 / Hkv=8, D=128): per-head
-    RMSNorm + RoPE of Q, and the K/V page write into FP8 pages.  Both are HBM bound; bytes are what the kernel must move."""
+    """The kernels that feed the SDPA, at config 5's prefill shape (8 x 2048 new tokens, Hq=64 / Hkv=8, D=128): per-head
+    RMSNorm + RoPE of Q, the K/V page write into FP8 pages, and K RMSNorm + RoPE fused with that write.  All are HBM bound;
+    bytes are what the kernel must move."""
     import torch
 
     from khalamari_amd import kv_page_write, rms_norm_rope
@@ -515,6 +516,26 @@ def producer_rows(device, steps: int = 20) -> dict:
     nbytes = 2 * flat_k.numel() * 2 + 2 * flat_k.numel()
     result["kv_page_write"] = {"workload": f"K/V rows {tokens}x{hkv}x{d} bf16 -> FP8 E4M3FN pages", "kernel_us": us, "algorithmic_bytes": nbytes,
                                "gbps": nbytes / us / 1e3, "roofline_frac": nbytes / us / 1e3 / HBM_PEAK_GBPS}
+
+    # K RMSNorm + RoPE and the page write in one launch, beside the two launches it replaces (K norm/rope, then the writer)
+    from khalamari_amd import k_norm_rope_page_write
+
+    k_norm = rms_norm_rope.Compute(rms_norm_rope.Config.bf16(hkv, d, d, 1e-6, 1_000_000.0))
+    k_rows = torch.empty_like(flat_k)
+
+    def two_launches():
+        k_norm.invoke(rms_norm_rope.Shape(tokens), input=flat_k, norm_weight=weight, flat_token_indices=positions, output=k_rows,
+                      num_active_tokens=ReplayU32.fixed(tokens))
+        writer.invoke(shape, pages=pages, flat_k=k_rows, flat_v=flat_v, req_slots=req_slots, flat_token_indices=positions, page_ids=page_ids,
+                      num_active_token_writes=ReplayU32.fixed(tokens), page_table_index=ReplayU32.fixed(0))
+
+    fused = k_norm_rope_page_write.Compute(rms_norm_rope.Config.bf16(hkv, d, d, 1e-6, 1_000_000.0), kv_page_write.Config(hkv, d, page_bytes))
+    separate_us = timed(two_launches)
+    us = timed(lambda: fused.invoke(shape, pages=pages, k=flat_k, v=flat_v, norm_weight=weight, req_slots=req_slots, flat_token_indices=positions,
+                                    page_ids=page_ids, num_active_tokens=ReplayU32.fixed(tokens), page_table_index=ReplayU32.fixed(0)))
+    result["k_norm_rope_page_write"] = {"workload": f"K RMSNorm + RoPE and K/V rows {tokens}x{hkv}x{d} bf16 -> FP8 E4M3FN pages, one launch",
+                                        "kernel_us": us, "algorithmic_bytes": nbytes, "gbps": nbytes / us / 1e3,
+                                        "roofline_frac": nbytes / us / 1e3 / HBM_PEAK_GBPS, "two_launches_us": separate_us}
     return result
 
 

@@ -473,6 +473,27 @@ int khm_rms_norm_rope_kernel_parameters(const khm_rms_norm_rope_config* config, 
 int khm_rms_norm_rope(const khm_rms_norm_rope_config* config, uint32_t num_total_tokens, const khm_rms_norm_rope_buffers* buffers,
                       khm_replay_u32 num_active_tokens, const uint32_t* replay_parameters, void* stream);
 
+/* K RMSNorm + RoPE fused with the K/V page write: what GQA::record enqueues as k_norm_rope -> scratch.k_norm_rope ->
+ * kv_page_write (crates/inference-executor-metal/src/attn/gqa/backend.rs:382-412; rms_norm_rope.rs:286-403,
+ * kv_page_write.rs:136-262) as one launch without the bf16 K round trip through memory.  The pages receive exactly the
+ * bytes the two calls would have written.  norm_config.num_heads / head_dim must equal page_config.num_kv_heads /
+ * head_dim and norm_config.dtype must be BF16; flat_token_indices are both the rotary positions and the token slots of
+ * the writes, as in the reference.  KHM_ERR_UNSUPPORTED for shapes outside the vector path (head_dim > 512, head_dim or
+ * rope_dim / 2 no multiple of 8, buffers not 16-byte aligned): the two separate calls cover those. */
+typedef struct khm_k_norm_rope_page_write_buffers {
+    khm_buffer pages;
+    khm_buffer k;           /* bf16 [W][Hkv][D], before the norm */
+    khm_buffer v;           /* bf16 [W][Hkv][D] */
+    khm_buffer norm_weight; /* [D], norm_config.norm_weight_dtype */
+    khm_buffer req_slots;
+    khm_buffer flat_token_indices;
+    khm_buffer page_ids;
+} khm_k_norm_rope_page_write_buffers;
+int khm_k_norm_rope_page_write(const khm_rms_norm_rope_config* norm_config, const khm_kv_page_write_config* page_config,
+                               const khm_kv_page_write_shape* shape, const khm_k_norm_rope_page_write_buffers* buffers,
+                               khm_replay_u32 num_active_tokens, khm_replay_u32 page_table_index,
+                               const uint32_t* replay_parameters, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Executor-side host logic that feeds the component (CPU only, no HIP calls)
  * ------------------------------------------------------------------------------------------ */

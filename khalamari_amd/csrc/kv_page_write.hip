@@ -12,27 +12,10 @@
 #include "device_math.hip.h"
 #include "device_params.h"
 #include "fp8_device.hip.h"
+#include "page_write_params.h"
 
 namespace khm {
 
-struct PageWriteParams {
-    uint8_t* pages;
-    const uint16_t* flat_k;             // bf16 [W][Hkv][D]
-    const uint16_t* flat_v;
-    const uint32_t* req_slots;          // [W]
-    const uint32_t* flat_token_indices; // [W]
-    const uint32_t* page_ids;           // [R][L][NB][PPB]
-    const uint32_t* replay_parameters;
-    DeviceReplayU32 num_active_token_writes;
-    DeviceReplayU32 layer_index;
-    uint64_t page_bytes;
-    uint32_t num_kv_heads;
-    uint32_t head_dim;
-    uint32_t tokens_per_page;
-    uint32_t num_gqa_layers;
-    uint32_t num_blocks;
-    uint32_t num_page_ids_per_block;
-};
 
 // A block serves one token write (blockIdx.x), so the request slot, the page-table walk and the page address are
 // wave-uniform scalar work; a thread moves eight consecutive dims of one KV head's row, for K and for V: a 16-byte load
@@ -51,17 +34,10 @@ __global__ __launch_bounds__(1024) void kv_page_write_kernel(const PageWritePara
     const uint32_t req_slot = p.req_slots[write_index];
     const uint32_t token = p.flat_token_indices[write_index];
     const uint32_t layer = resolve_u32(p.layer_index, p.replay_parameters);
-    const uint32_t block = token / (p.tokens_per_page * p.num_page_ids_per_block);
-    const uint32_t page_index = (token / p.tokens_per_page) % p.num_page_ids_per_block;
-    const uint64_t table_index = (((uint64_t)req_slot * p.num_gqa_layers + layer) * p.num_blocks + block) * p.num_page_ids_per_block + page_index;
-    const uint64_t page_id = p.page_ids[table_index];
-    const uint32_t page_token = token % p.tokens_per_page;
-
     constexpr uint32_t kElementBytes = FP8_PAGES ? 1 : 2;
-    const uint64_t values_per_plane = (uint64_t)p.num_kv_heads * p.tokens_per_page * p.head_dim;
-    const uint64_t in_plane = ((uint64_t)head * p.tokens_per_page + page_token) * p.head_dim + dim;
-    uint8_t* k_target = p.pages + page_id * p.page_bytes + in_plane * kElementBytes;
-    uint8_t* v_target = k_target + values_per_plane * kElementBytes;
+    const PageTarget target = page_target_of(p, req_slot, token, layer, head, dim, kElementBytes);
+    uint8_t* k_target = p.pages + target.k_offset;
+    uint8_t* v_target = k_target + target.v_distance;
     const uint64_t source = ((uint64_t)write_index * p.num_kv_heads + head) * p.head_dim + dim;
 
     if (dim + 8 <= p.head_dim && p.head_dim % 8 == 0) {
@@ -138,10 +114,10 @@ extern "C" uint32_t khm_kv_page_write_num_tokens_per_page(const khm_kv_page_writ
     return (uint32_t)(config->page_bytes / bytes_per_token);
 }
 
-extern "C" int khm_kv_page_write(const khm_kv_page_write_config* config, const khm_kv_page_write_shape* shape,
-                                 const khm_kv_page_write_buffers* buffers, khm_replay_u32 num_active_token_writes,
-                                 khm_replay_u32 page_table_index, const uint32_t* replay_parameters, void* stream) {
-    clear_error();
+// see page_write_params.h
+int khm::fill_page_write_params(const khm_kv_page_write_config* config, const khm_kv_page_write_shape* shape,
+                                const khm_kv_page_write_buffers* buffers, khm_replay_u32 num_active_token_writes,
+                                khm_replay_u32 page_table_index, const uint32_t* replay_parameters, PageWriteParams* out) {
     KHM_REQUIRE(config != nullptr && shape != nullptr && buffers != nullptr, "config, shape and buffers must not be null");
     // Config::validate (kv_page_write.rs:67-75)
     KHM_REQUIRE(config->num_kv_heads > 0, "GQA KV page write requires KV heads");
@@ -205,6 +181,16 @@ extern "C" int khm_kv_page_write(const khm_kv_page_write_config* config, const k
     p.num_gqa_layers = layout.num_gqa_layers;
     p.num_blocks = layout.num_blocks;
     p.num_page_ids_per_block = layout.num_page_ids_per_block;
+    *out = p;
+    return KHM_OK;
+}
+
+extern "C" int khm_kv_page_write(const khm_kv_page_write_config* config, const khm_kv_page_write_shape* shape,
+                                 const khm_kv_page_write_buffers* buffers, khm_replay_u32 num_active_token_writes,
+                                 khm_replay_u32 page_table_index, const uint32_t* replay_parameters, void* stream) {
+    clear_error();
+    PageWriteParams p{};
+    if (int status = fill_page_write_params(config, shape, buffers, num_active_token_writes, page_table_index, replay_parameters, &p)) return status;
     const uint64_t chunks_per_write = (uint64_t)config->num_kv_heads * ((config->head_dim + 7) / 8);
     const uint32_t block_threads = (uint32_t)(chunks_per_write >= 1024 ? 1024 : (chunks_per_write + 63) / 64 * 64);
     const uint64_t chunk_blocks = (chunks_per_write + block_threads - 1) / block_threads;

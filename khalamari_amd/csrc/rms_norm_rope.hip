@@ -7,12 +7,16 @@
 // computed on the host per call and travels as a kernel argument, so nothing is allocated.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
+#include <type_traits>
 #include <vector>
 
 #include "common.h"
 #include "device_math.hip.h"
 #include "device_params.h"
+#include "fp8_device.hip.h"
+#include "page_write_params.h"
 
 namespace khm {
 
@@ -30,6 +34,8 @@ struct RmsNormRopeParams {
     uint32_t rope_dim;
     float eps;
     float attention_factor;
+    uint32_t tokens_per_block;      // rows kernels: tokens a block serves (more than one when there are few heads)
+    uint32_t row_slots_per_token_shift;  // rows kernels: log2 of the row slots of a block that one token takes
     float inverse_frequencies[kMaxRopeHalf];
 };
 
@@ -158,15 +164,25 @@ __device__ __forceinline__ float sum_in_row(float v, uint32_t lane) {
 // of ONE token: the first lanes evaluate the token's sines and cosines once into LDS, and each wave issues the loads
 // of up to kRowsInFlight row groups before it uses the first.
 constexpr int kRowsInFlight = 4;
+constexpr int kMaxTokensPerBlock = 16;
 
-template <typename T, typename W, uint32_t LPR, uint32_t PARTNER>
-__global__ __launch_bounds__(256) void rms_norm_rope_rows_kernel(const RmsNormRopeParams p) {
+// PAGES: 0 writes the rows to p.output; 1 / 2 scatter them, as K rows, straight into bf16 / FP8 E4M3FN pages through
+// the page table and copy the V rows of the same (token, KV head) beside them: RMSNorm + RoPE of K and the K/V page write
+// in one pass, the bf16 value the two-kernel sequence would have stored in between being the one that is encoded.
+template <typename T, typename W, uint32_t LPR, uint32_t PARTNER, int PAGES>
+__device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, const PageWriteParams* pages) {
+    static_assert(PAGES == 0 || sizeof(T) == 2, "pages are written from bf16 rows");
     constexpr uint32_t kRowsPerWave = 64u / LPR;
-    constexpr uint32_t kHeadsPerBlock = 4 * kRowsInFlight * kRowsPerWave;
+    constexpr uint32_t kRowSlots = 4 * kRowsInFlight * kRowsPerWave;   // (token, head) rows a block holds
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
-    const uint32_t token = blockIdx.x;
-    if (token >= resolve_u32(p.num_active_tokens, p.replay_parameters)) return;
+    // Row slot s of the block belongs to token s >> shift of the block's tokens and to head s & (2^shift - 1) of this
+    // block's head group: one token per block when the heads fill the slots, several when there are few heads (the K
+    // rows of a grouped-query model), so that every wave has rows and a token's sines and cosines are shared by its heads.
+    const uint32_t tokens_per_block = p.tokens_per_block, slot_shift = p.row_slots_per_token_shift;
+    const uint32_t num_active_tokens = resolve_u32(p.num_active_tokens, p.replay_parameters);
+    const uint32_t first_token = blockIdx.x * tokens_per_block;
+    if (first_token >= num_active_tokens) return;
     const uint32_t sub_row = lane / LPR;
     const uint32_t first = (lane % LPR) * 8;
     const bool holds = first < p.head_dim;
@@ -175,32 +191,46 @@ __global__ __launch_bounds__(256) void rms_norm_rope_rows_kernel(const RmsNormRo
     const int partner_lane = ((int)lane + (lower ? (int)(rope_half / 8) : -(int)(rope_half / 8))) & 63;
 
     float x[kRowsInFlight][8];
-    uint32_t heads[kRowsInFlight];
+    uint32_t heads[kRowsInFlight], tokens[kRowsInFlight], local_tokens[kRowsInFlight];
+    bool valid[kRowsInFlight];
 #pragma unroll
     for (int j = 0; j < kRowsInFlight; ++j) {
-        heads[j] = blockIdx.y * kHeadsPerBlock + (j * 4 + wave) * kRowsPerWave + sub_row;
+        const uint32_t slot = (j * 4 + wave) * kRowsPerWave + sub_row;
+        local_tokens[j] = slot >> slot_shift;
+        tokens[j] = first_token + local_tokens[j];
+        heads[j] = blockIdx.y * kRowSlots + (slot & ((1u << slot_shift) - 1u));
+        valid[j] = holds && heads[j] < p.num_heads && local_tokens[j] < tokens_per_block && tokens[j] < num_active_tokens;
 #pragma unroll
         for (int i = 0; i < 8; ++i) x[j][i] = 0.0f;
-        if (holds && heads[j] < p.num_heads) Row8<T>::load(static_cast<const T*>(p.input) + ((uint64_t)token * p.num_heads + heads[j]) * p.head_dim + first, x[j]);
+        if (valid[j]) Row8<T>::load(static_cast<const T*>(p.input) + ((uint64_t)tokens[j] * p.num_heads + heads[j]) * p.head_dim + first, x[j]);
     }
-    // the token's rotation table, one sine/cosine evaluation per rotary pair for the whole block
-    __shared__ __align__(16) float sines[kMaxRopeHalf];
-    __shared__ __align__(16) float cosines[kMaxRopeHalf];
-    if (threadIdx.x < rope_half) {
-        const float position = (float)p.flat_token_indices[token];
-        sincosf(position * p.inverse_frequencies[threadIdx.x], &sines[threadIdx.x], &cosines[threadIdx.x]);
-    }
-    float w[8], sine[8], cosine[8];
+    uint4 v_chunk[PAGES != 0 ? kRowsInFlight : 1];
+    if constexpr (PAGES != 0) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) w[i] = 0.0f, sine[i] = 0.0f, cosine[i] = 1.0f;
+        for (int j = 0; j < kRowsInFlight; ++j) {
+            v_chunk[j] = make_uint4(0, 0, 0, 0);
+            if (valid[j]) v_chunk[j] = *reinterpret_cast<const uint4*>(pages->flat_v + ((uint64_t)tokens[j] * p.num_heads + heads[j]) * p.head_dim + first);
+        }
+    }
+    // the rotation tables of the block's tokens, one sine/cosine evaluation per token and rotary pair
+    __shared__ __align__(16) float sines[kMaxTokensPerBlock * kMaxRopeHalf];
+    __shared__ __align__(16) float cosines[kMaxTokensPerBlock * kMaxRopeHalf];
+    for (uint32_t entry = threadIdx.x; entry < tokens_per_block * rope_half; entry += 256) {
+        const uint32_t local = entry / rope_half, pair = entry - local * rope_half;
+        if (first_token + local < num_active_tokens) {
+            const float position = (float)p.flat_token_indices[first_token + local];
+            sincosf(position * p.inverse_frequencies[pair], &sines[local * rope_half + pair], &cosines[local * rope_half + pair]);
+        }
+    }
+    float w[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w[i] = 0.0f;
     if (holds) Row8<W>::load(static_cast<const W*>(p.norm_weight) + first, w);
     __syncthreads();
-    if (rotated) {
-        const uint32_t pair = lower ? first : first - rope_half;
-        Row8<float>::load(sines + pair, sine);
-        Row8<float>::load(cosines + pair, cosine);
-    }
     const float inverse_dim = 1.0f / (float)p.head_dim;
+    float sine[8], cosine[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sine[i] = 0.0f, cosine[i] = 1.0f;
 #pragma unroll
     for (int j = 0; j < kRowsInFlight; ++j) {
         float acc = 0.0f;
@@ -211,6 +241,11 @@ __global__ __launch_bounds__(256) void rms_norm_rope_rows_kernel(const RmsNormRo
         const float mean = acc * inverse_dim + p.eps;
         float inv_rms = __builtin_amdgcn_rsqf(mean);
         inv_rms = inv_rms * __builtin_fmaf(-0.5f * mean * inv_rms, inv_rms, 1.5f);
+        if (rotated && valid[j] && (j == 0 || tokens_per_block > 1)) {   // one token per block: every row shares the first load
+            const uint32_t pair = local_tokens[j] * rope_half + (lower ? first : first - rope_half);
+            Row8<float>::load(sines + pair, sine);
+            Row8<float>::load(cosines + pair, cosine);
+        }
         float out[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -231,8 +266,38 @@ __global__ __launch_bounds__(256) void rms_norm_rope_rows_kernel(const RmsNormRo
                                : p.attention_factor * (partner * sine[i] + normed * cosine[i]);
             }
         }
-        if (holds && heads[j] < p.num_heads) Row8<T>::store(static_cast<T*>(p.output) + ((uint64_t)token * p.num_heads + heads[j]) * p.head_dim + first, out);
+        if (!valid[j]) continue;
+        if constexpr (PAGES == 0) {
+            Row8<T>::store(static_cast<T*>(p.output) + ((uint64_t)tokens[j] * p.num_heads + heads[j]) * p.head_dim + first, out);
+        } else {
+            const uint4 k_chunk = make_uint4(pack_bf16x2(out[0], out[1]), pack_bf16x2(out[2], out[3]), pack_bf16x2(out[4], out[5]), pack_bf16x2(out[6], out[7]));
+            constexpr uint32_t kElementBytes = PAGES == 2 ? 1 : 2;
+            const PageTarget target = page_target_of(*pages, pages->req_slots[tokens[j]], pages->flat_token_indices[tokens[j]],
+                                                     resolve_u32(pages->layer_index, pages->replay_parameters), heads[j], first, kElementBytes);
+            uint8_t* k_target = pages->pages + target.k_offset;
+            if constexpr (PAGES == 2) {
+                auto encode8 = [](uint4 bits) {
+                    return make_uint2(bf16x2_bits_to_fp8x2_e4m3fn(bits.x) | (bf16x2_bits_to_fp8x2_e4m3fn(bits.y) << 16),
+                                      bf16x2_bits_to_fp8x2_e4m3fn(bits.z) | (bf16x2_bits_to_fp8x2_e4m3fn(bits.w) << 16));
+                };
+                *reinterpret_cast<uint2*>(k_target) = encode8(k_chunk);
+                *reinterpret_cast<uint2*>(k_target + target.v_distance) = encode8(v_chunk[j]);
+            } else {
+                *reinterpret_cast<uint4*>(k_target) = k_chunk;
+                *reinterpret_cast<uint4*>(k_target + target.v_distance) = v_chunk[j];
+            }
+        }
     }
+}
+
+template <typename T, typename W, uint32_t LPR, uint32_t PARTNER>
+__global__ __launch_bounds__(256) void rms_norm_rope_rows_kernel(const RmsNormRopeParams p) {
+    rms_norm_rope_rows<T, W, LPR, PARTNER, 0>(p, nullptr);
+}
+
+template <typename W, uint32_t LPR, uint32_t PARTNER, bool FP8_PAGES>
+__global__ __launch_bounds__(256) void k_norm_rope_page_write_kernel(const RmsNormRopeParams p, const PageWriteParams pages) {
+    rms_norm_rope_rows<uint16_t, W, LPR, PARTNER, FP8_PAGES ? 2 : 1>(p, &pages);
 }
 
 // RopeScaling::yarn_kernel_parameters (rms_norm_rope.rs:206-243).
@@ -328,11 +393,12 @@ extern "C" int khm_rms_norm_rope_kernel_parameters(const khm_rms_norm_rope_confi
     return KHM_OK;
 }
 
-extern "C" int khm_rms_norm_rope(const khm_rms_norm_rope_config* config, uint32_t num_total_tokens, const khm_rms_norm_rope_buffers* buffers,
-                                 khm_replay_u32 num_active_tokens, const uint32_t* replay_parameters, void* stream) {
-    clear_error();
+// Config / Shape / Invocation validation of one RMSNorm/RoPE call and its kernel arguments; `output` may be absent when
+// the rows go elsewhere (the fused page write).
+static int fill_rms_norm_rope_params(const khm_rms_norm_rope_config* config, uint32_t num_total_tokens, const khm_buffer& input,
+                                     const khm_buffer& norm_weight, const khm_buffer& flat_token_indices, const khm_buffer* output,
+                                     khm_replay_u32 num_active_tokens, const uint32_t* replay_parameters, RmsNormRopeParams* out) {
     if (int status = validate_rms_norm_rope_config(config)) return status;
-    KHM_REQUIRE(buffers != nullptr, "buffers must not be null");
     KHM_REQUIRE(config->rope_dim / 2 <= (uint32_t)kMaxRopeHalf, "gfx950 RMSNorm/RoPE holds at most %d rotary pairs", kMaxRopeHalf);
     // Shape::validate (rms_norm_rope.rs:278-284)
     KHM_REQUIRE(num_total_tokens > 0, "RMSNorm/RoPE requires tokens");
@@ -351,45 +417,79 @@ extern "C" int khm_rms_norm_rope(const khm_rms_norm_rope_config* config, uint32_
 #define KHM_NORM_AT_LEAST(buffer, need, name)                                                                                  \
     KHM_REQUIRE((buffer).ptr != nullptr && (buffer).len_bytes >= (uint64_t)(need), "%s buffer holds %llu bytes, needs %llu", name, \
                 (unsigned long long)(buffer).len_bytes, (unsigned long long)(need))
-    KHM_NORM_AT_LEAST(buffers->input, bytes, "input");
-    KHM_NORM_AT_LEAST(buffers->norm_weight, weight_bytes, "norm_weight");
-    KHM_NORM_AT_LEAST(buffers->flat_token_indices, (uint64_t)num_total_tokens * 4, "flat_token_indices");
-    KHM_NORM_AT_LEAST(buffers->output, bytes, "output");
+    KHM_NORM_AT_LEAST(input, bytes, "input");
+    KHM_NORM_AT_LEAST(norm_weight, weight_bytes, "norm_weight");
+    KHM_NORM_AT_LEAST(flat_token_indices, (uint64_t)num_total_tokens * 4, "flat_token_indices");
+    if (output != nullptr) KHM_NORM_AT_LEAST(*output, bytes, "output");
 #undef KHM_NORM_AT_LEAST
 
     RmsNormRopeParams p{};
     if (int status = rope_kernel_parameters(*config, p.inverse_frequencies, &p.attention_factor)) return status;
-    p.input = buffers->input.ptr;
-    p.norm_weight = buffers->norm_weight.ptr;
-    p.flat_token_indices = static_cast<const uint32_t*>(buffers->flat_token_indices.ptr);
-    p.output = buffers->output.ptr;
+    p.input = input.ptr;
+    p.norm_weight = norm_weight.ptr;
+    p.flat_token_indices = static_cast<const uint32_t*>(flat_token_indices.ptr);
+    p.output = output != nullptr ? output->ptr : nullptr;
     p.replay_parameters = replay_parameters;
     p.num_active_tokens = DeviceReplayU32{num_active_tokens.is_parameter, num_active_tokens.value};
     p.num_heads = config->num_heads;
     p.head_dim = config->head_dim;
     p.rope_dim = config->rope_dim;
     p.eps = config->eps;
+    *out = p;
+    return KHM_OK;
+}
+
+// Launch geometry of the rows kernels: lanes per row, the lane distance of a rotary pair when a vector exchange reaches
+// it (0 otherwise), and the grid (one block per token and group of heads).
+struct RowsGeometry {
+    bool fits;   // vector loads need 16-byte aligned rows; head_dim <= 512, head_dim and rope_dim / 2 multiples of 8
+    uint32_t lanes_per_row, partner, tokens_per_block, slot_shift;
+    dim3 grid;
+};
+static RowsGeometry rows_geometry(const khm_rms_norm_rope_config& config, uint32_t num_total_tokens, uintptr_t address_bits) {
+    RowsGeometry g{};
+    g.fits = address_bits % 16 == 0 && config.head_dim <= 512 && config.head_dim % 8 == 0 && (config.rope_dim / 2) % 8 == 0;
+    g.lanes_per_row = config.head_dim <= 64 ? 8u : (config.head_dim <= 128 ? 16u : (config.head_dim <= 256 ? 32u : 64u));
+    const uint32_t row_slots = 4 * kRowsInFlight * (64u / g.lanes_per_row);   // a power of two
+    // few heads: a token takes the next power of two of row slots and a block serves several tokens
+    uint32_t slots_per_token = 1;
+    while (slots_per_token < config.num_heads && slots_per_token < row_slots) slots_per_token *= 2;
+    g.tokens_per_block = std::min<uint32_t>(row_slots / slots_per_token, (uint32_t)kMaxTokensPerBlock);
+    g.slot_shift = 0;
+    while ((1u << g.slot_shift) < slots_per_token) ++g.slot_shift;
+    g.grid = dim3((num_total_tokens + g.tokens_per_block - 1) / g.tokens_per_block, (config.num_heads + row_slots - 1) / row_slots);
+    const uint32_t partner_distance = config.rope_dim / 16;   // lanes between the halves of a rotary pair
+    const bool vector_partner = partner_distance == 8 || partner_distance == 16 || partner_distance == 32;
+    g.partner = vector_partner && partner_distance < g.lanes_per_row ? partner_distance : 0;
+    return g;
+}
+
+#define KHM_ROWS_CASES(CASE) \
+    CASE(8, 0) CASE(16, 0) CASE(16, 8) CASE(32, 0) CASE(32, 8) CASE(32, 16) CASE(64, 0) CASE(64, 8) CASE(64, 16) CASE(64, 32)
+
+extern "C" int khm_rms_norm_rope(const khm_rms_norm_rope_config* config, uint32_t num_total_tokens, const khm_rms_norm_rope_buffers* buffers,
+                                 khm_replay_u32 num_active_tokens, const uint32_t* replay_parameters, void* stream) {
+    clear_error();
+    KHM_REQUIRE(buffers != nullptr, "buffers must not be null");
+    RmsNormRopeParams p{};
+    if (int status = fill_rms_norm_rope_params(config, num_total_tokens, buffers->input, buffers->norm_weight, buffers->flat_token_indices,
+                                               &buffers->output, num_active_tokens, replay_parameters, &p))
+        return status;
     hipStream_t hip_stream = static_cast<hipStream_t>(stream);
     const bool io_bf16 = config->dtype == KHM_DTYPE_BF16, weight_bf16 = config->norm_weight_dtype == KHM_DTYPE_BF16;
-    // vector loads need 16-byte aligned rows; allocator-aligned bases and head_dim % 8 == 0 give that
-    const bool aligned = ((uintptr_t)p.input | (uintptr_t)p.output | (uintptr_t)p.norm_weight) % 16 == 0;
-    if (aligned && config->head_dim <= 512 && config->head_dim % 8 == 0 && (config->rope_dim / 2) % 8 == 0) {
-        const uint32_t lanes_per_row = config->head_dim <= 64 ? 8u : (config->head_dim <= 128 ? 16u : (config->head_dim <= 256 ? 32u : 64u));
-        const uint32_t heads_per_block = 4 * kRowsInFlight * (64u / lanes_per_row);
-        const dim3 grid(num_total_tokens, (config->num_heads + heads_per_block - 1) / heads_per_block);
-        const uint32_t partner_distance = config->rope_dim / 16;   // lanes between the halves of a rotary pair
-        const bool vector_partner = partner_distance == 8 || partner_distance == 16 || partner_distance == 32;
-        const uint32_t partner = vector_partner && partner_distance < lanes_per_row ? partner_distance : 0;
+    const RowsGeometry geometry = rows_geometry(*config, num_total_tokens, (uintptr_t)p.input | (uintptr_t)p.output | (uintptr_t)p.norm_weight);
+    p.tokens_per_block = geometry.tokens_per_block;
+    p.row_slots_per_token_shift = geometry.slot_shift;
+    if (geometry.fits) {
         auto launch = [&](auto io_tag, auto weight_tag) {
             typedef decltype(io_tag) T;
             typedef decltype(weight_tag) W;
 #define KHM_ROWS_CASE(LPR, PARTNER)                                                                                        \
-    if (lanes_per_row == LPR && partner == PARTNER) {                                                                      \
-        hipLaunchKernelGGL((rms_norm_rope_rows_kernel<T, W, LPR, PARTNER>), grid, dim3(256), 0, hip_stream, p);             \
+    if (geometry.lanes_per_row == LPR && geometry.partner == PARTNER) {                                                    \
+        hipLaunchKernelGGL((rms_norm_rope_rows_kernel<T, W, LPR, PARTNER>), geometry.grid, dim3(256), 0, hip_stream, p);    \
         return;                                                                                                            \
     }
-            KHM_ROWS_CASE(8, 0) KHM_ROWS_CASE(16, 0) KHM_ROWS_CASE(16, 8) KHM_ROWS_CASE(32, 0) KHM_ROWS_CASE(32, 8) KHM_ROWS_CASE(32, 16)
-            KHM_ROWS_CASE(64, 0) KHM_ROWS_CASE(64, 8) KHM_ROWS_CASE(64, 16) KHM_ROWS_CASE(64, 32)
+            KHM_ROWS_CASES(KHM_ROWS_CASE)
 #undef KHM_ROWS_CASE
         };
         if (io_bf16 && weight_bf16) launch(uint16_t{}, uint16_t{});
@@ -397,7 +497,7 @@ extern "C" int khm_rms_norm_rope(const khm_rms_norm_rope_config* config, uint32_
         else if (weight_bf16) launch(float{}, uint16_t{});
         else launch(float{}, float{});
     } else {
-        const dim3 grid((uint32_t)rows);
+        const dim3 grid(num_total_tokens * config->num_heads);
         if (io_bf16 && weight_bf16) hipLaunchKernelGGL((rms_norm_rope_kernel<uint16_t, uint16_t>), grid, dim3(64), 0, hip_stream, p);
         else if (io_bf16) hipLaunchKernelGGL((rms_norm_rope_kernel<uint16_t, float>), grid, dim3(64), 0, hip_stream, p);
         else if (weight_bf16) hipLaunchKernelGGL((rms_norm_rope_kernel<float, uint16_t>), grid, dim3(64), 0, hip_stream, p);
@@ -405,5 +505,57 @@ extern "C" int khm_rms_norm_rope(const khm_rms_norm_rope_config* config, uint32_
     }
     const hipError_t status = hipGetLastError();
     if (status != hipSuccess) return fail(KHM_ERR_HIP, "RMSNorm/RoPE launch failed: %s", hipGetErrorString(status));
+    return KHM_OK;
+}
+
+// K RMSNorm + RoPE and the K/V page write in one launch (the reference records k_norm_rope -> scratch.k_norm_rope ->
+// kv_page_write: crates/inference-executor-metal/src/attn/gqa/backend.rs:382-412): the normalized, rotated K row is
+// rounded to bf16 exactly as the first kernel would store it and goes straight into its page, V is copied beside it.
+extern "C" int khm_k_norm_rope_page_write(const khm_rms_norm_rope_config* norm_config, const khm_kv_page_write_config* page_config,
+                                          const khm_kv_page_write_shape* shape, const khm_k_norm_rope_page_write_buffers* buffers,
+                                          khm_replay_u32 num_active_tokens, khm_replay_u32 page_table_index,
+                                          const uint32_t* replay_parameters, void* stream) {
+    clear_error();
+    KHM_REQUIRE(norm_config != nullptr && page_config != nullptr && shape != nullptr && buffers != nullptr,
+                "configs, shape and buffers must not be null");
+    KHM_REQUIRE(norm_config->num_heads == page_config->num_kv_heads && norm_config->head_dim == page_config->head_dim,
+                "K RMSNorm/RoPE rows [%u][%u] do not match the page writer's KV heads [%u][%u]", norm_config->num_heads,
+                norm_config->head_dim, page_config->num_kv_heads, page_config->head_dim);
+    KHM_REQUIRE(norm_config->dtype == KHM_DTYPE_BF16, "the fused K RMSNorm/RoPE page write takes BF16 K and V rows");
+    const khm_kv_page_write_buffers page_buffers{buffers->pages, buffers->k, buffers->v, buffers->req_slots, buffers->flat_token_indices,
+                                                 buffers->page_ids};
+    PageWriteParams pages{};
+    if (int status = fill_page_write_params(page_config, shape, &page_buffers, num_active_tokens, page_table_index, replay_parameters, &pages))
+        return status;
+    RmsNormRopeParams p{};
+    if (int status = fill_rms_norm_rope_params(norm_config, shape->num_total_token_writes, buffers->k, buffers->norm_weight,
+                                               buffers->flat_token_indices, nullptr, num_active_tokens, replay_parameters, &p))
+        return status;
+    const RowsGeometry geometry = rows_geometry(*norm_config, shape->num_total_token_writes,
+                                                (uintptr_t)p.input | (uintptr_t)pages.flat_v | (uintptr_t)p.norm_weight | (uintptr_t)pages.pages);
+    if (!geometry.fits || page_config->page_bytes % 16 != 0)
+        return fail(KHM_ERR_UNSUPPORTED, "the fused K RMSNorm/RoPE page write needs 16-byte aligned buffers, head_dim <= 512, and head_dim and "
+                                         "rope_dim / 2 multiples of 8: run khm_rms_norm_rope and khm_kv_page_write instead");
+    p.tokens_per_block = geometry.tokens_per_block;
+    p.row_slots_per_token_shift = geometry.slot_shift;
+    hipStream_t hip_stream = static_cast<hipStream_t>(stream);
+    const bool weight_bf16 = norm_config->norm_weight_dtype == KHM_DTYPE_BF16, fp8_pages = page_config->kv_dtype == KHM_DTYPE_FP8_E4M3FN;
+    auto launch = [&](auto weight_tag, auto fp8_tag) {
+        typedef decltype(weight_tag) W;
+        constexpr bool FP8 = decltype(fp8_tag)::value;
+#define KHM_ROWS_CASE(LPR, PARTNER)                                                                                                    \
+    if (geometry.lanes_per_row == LPR && geometry.partner == PARTNER) {                                                                \
+        hipLaunchKernelGGL((k_norm_rope_page_write_kernel<W, LPR, PARTNER, FP8>), geometry.grid, dim3(256), 0, hip_stream, p, pages);   \
+        return;                                                                                                                        \
+    }
+        KHM_ROWS_CASES(KHM_ROWS_CASE)
+#undef KHM_ROWS_CASE
+    };
+    if (weight_bf16 && fp8_pages) launch(uint16_t{}, std::true_type{});
+    else if (weight_bf16) launch(uint16_t{}, std::false_type{});
+    else if (fp8_pages) launch(float{}, std::true_type{});
+    else launch(float{}, std::false_type{});
+    const hipError_t status = hipGetLastError();
+    if (status != hipSuccess) return fail(KHM_ERR_HIP, "K RMSNorm/RoPE page write launch failed: %s", hipGetErrorString(status));
     return KHM_OK;
 }
