@@ -323,6 +323,16 @@ int khm_sliced_q_direct(const khm_sliced_q* compute, const khm_sliced_q_direct_b
 /* Compute::invoke_reduce + ReduceInvocation::record (sliced_q.rs:484-504,620-642). */
 int khm_sliced_q_reduce(const khm_sliced_q* compute, const khm_sliced_q_reduce_buffers* buffers,
                         khm_replay_u32 num_active_q_token_tiles, const uint32_t* replay_parameters, void* stream);
+/* The same two calls fused with the sigmoid gate that follows the SDPA in GQA::record
+ * (crates/inference-executor-metal/src/attn/gqa/backend.rs:413-421; activation_gate.rs:35-168,
+ * gqa_activation_gate.metal:19-39): output = bf16(attn) * sigmoid(gate) with the kernel's bf16 step rounding, so the
+ * result equals khm_sliced_q_direct / khm_sliced_q_reduce followed by khm_gqa_activation_gate bit for bit, without the
+ * extra pass over the output.  gates: bf16 [T][Hq][D]. */
+int khm_sliced_q_direct_gated(const khm_sliced_q* compute, const khm_sliced_q_direct_buffers* buffers, khm_buffer gates,
+                              khm_replay_u32 page_table_index, khm_replay_u32 num_active_tokens,
+                              khm_replay_u32 num_active_q_token_tiles, const uint32_t* replay_parameters, void* stream);
+int khm_sliced_q_reduce_gated(const khm_sliced_q* compute, const khm_sliced_q_reduce_buffers* buffers, khm_buffer gates,
+                              khm_replay_u32 num_active_q_token_tiles, const uint32_t* replay_parameters, void* stream);
 
 /* Map and Reduce in one launch for the sliced-Q component; see khm_sliced_kv_map_reduce.
  *   arrival_counters  u32 [num_total_q_token_tiles][Hkv * q_head_ranges], zero before the first launch. */

@@ -246,6 +246,7 @@ EXPORTED_SYMBOLS = (
     "khm_sliced_kv_static_scratch_bytes", "khm_sliced_kv_map_reduce_static",
     "khm_sliced_q_partial_output_bytes", "khm_sliced_q_partial_output_stats_bytes", "khm_sliced_q_create",
     "khm_sliced_q_destroy", "khm_sliced_q_map_kernel_id", "khm_sliced_q_map", "khm_sliced_q_direct", "khm_sliced_q_reduce",
+    "khm_sliced_q_direct_gated", "khm_sliced_q_reduce_gated",
     "khm_sliced_q_arrival_counters_bytes", "khm_sliced_q_map_reduce",
     "khm_gqa_activation_gate",
     "khm_bf16_to_fp8_e4m3", "khm_fp8_e4m3_to_bf16", "khm_f32_to_bf16", "khm_bf16_to_f32",
@@ -330,6 +331,10 @@ def lib() -> ctypes.CDLL:
                                            ReplayU32, ctypes.c_void_p, ctypes.c_void_p]
     handle.khm_sliced_q_reduce.argtypes = [ctypes.c_void_p, ctypes.POINTER(SlicedQReduceBuffers), ReplayU32, ctypes.c_void_p,
                                            ctypes.c_void_p]
+    handle.khm_sliced_q_direct_gated.argtypes = [ctypes.c_void_p, ctypes.POINTER(SlicedQDirectBuffers), Buffer, ReplayU32, ReplayU32,
+                                                 ReplayU32, ctypes.c_void_p, ctypes.c_void_p]
+    handle.khm_sliced_q_reduce_gated.argtypes = [ctypes.c_void_p, ctypes.POINTER(SlicedQReduceBuffers), Buffer, ReplayU32, ctypes.c_void_p,
+                                                 ctypes.c_void_p]
     handle.khm_gqa_activation_gate.argtypes = [u32, u32, u32, u32, Buffer, Buffer, Buffer, ReplayU32, ctypes.c_void_p,
                                                ctypes.c_void_p]
     handle.khm_fp8_e4m3_to_bf16_device.argtypes = [Buffer, Buffer, u64, ctypes.c_void_p]

@@ -619,7 +619,7 @@ static int launch_sliced_q_map(const khm_sliced_q* compute, const khm_buffer& q,
                                const khm_buffer* maxs, const khm_buffer* output, khm_replay_u32 page_table_index,
                                khm_replay_u32 num_active_tokens, khm_replay_u32 num_active_q_token_tiles,
                                khm_replay_u32 num_active_kv_splits, const uint32_t* replay_parameters, void* stream,
-                               const FusedReduceArgs* fused = nullptr) {
+                               const FusedReduceArgs* fused = nullptr, const khm_buffer* direct_gates = nullptr) {
     const khm_gqa_sdpa_config& config = compute->config;
     const khm_gqa_sdpa_shape& shape = compute->shape;
     // MapInvocation::validate / DirectInvocation::validate (sliced_q.rs:519-545)
@@ -639,6 +639,10 @@ static int launch_sliced_q_map(const khm_sliced_q* compute, const khm_buffer& q,
         KHM_BUFFER_AT_LEAST(*output, khm_gqa_sdpa_q_bytes(&config, &shape), "output");
         p.out = output->ptr;
         p.output_mode = kMapDirectBf16;
+        if (direct_gates != nullptr) {
+            KHM_BUFFER_AT_LEAST(*direct_gates, khm_gqa_sdpa_q_bytes(&config, &shape), "gates");
+            p.gates = static_cast<const uint16_t*>(direct_gates->ptr);
+        }
     } else {
         KHM_BUFFER_AT_LEAST(*partial, khm_sliced_q_partial_output_bytes(&config, &compute->variant, &shape), "partial_output");
         KHM_BUFFER_AT_LEAST(*sums, khm_sliced_q_partial_output_stats_bytes(&config, &compute->variant, &shape), "partial_exp_sums");
@@ -725,9 +729,9 @@ extern "C" int khm_sliced_q_map(const khm_sliced_q* compute, const khm_sliced_q_
                                replay_parameters, stream);
 }
 
-extern "C" int khm_sliced_q_direct(const khm_sliced_q* compute, const khm_sliced_q_direct_buffers* buffers,
-                                   khm_replay_u32 page_table_index, khm_replay_u32 num_active_tokens,
-                                   khm_replay_u32 num_active_q_token_tiles, const uint32_t* replay_parameters, void* stream) {
+static int sliced_q_direct(const khm_sliced_q* compute, const khm_sliced_q_direct_buffers* buffers, const khm_buffer* gates,
+                           khm_replay_u32 page_table_index, khm_replay_u32 num_active_tokens,
+                           khm_replay_u32 num_active_q_token_tiles, const uint32_t* replay_parameters, void* stream) {
     clear_error();
     KHM_REQUIRE(compute != nullptr && buffers != nullptr, "compute and buffers must not be null");
     KHM_REQUIRE(compute->direct, "GQA SplitKV SlicedQ direct output requires a direct-output compute");
@@ -737,11 +741,23 @@ extern "C" int khm_sliced_q_direct(const khm_sliced_q* compute, const khm_sliced
     return launch_sliced_q_map(compute, buffers->q, buffers->kv_pages, buffers->req_slots, buffers->page_ids,
                                buffers->visible_kv_token_ranges, buffers->q_token_ranges, buffers->sdpa_map_task_templates, nullptr,
                                nullptr, nullptr, &buffers->output, page_table_index, num_active_tokens, num_active_q_token_tiles,
-                               num_active_q_token_tiles, replay_parameters, stream);
+                               num_active_q_token_tiles, replay_parameters, stream, nullptr, gates);
 }
 
-extern "C" int khm_sliced_q_reduce(const khm_sliced_q* compute, const khm_sliced_q_reduce_buffers* buffers,
+extern "C" int khm_sliced_q_direct(const khm_sliced_q* compute, const khm_sliced_q_direct_buffers* buffers,
+                                   khm_replay_u32 page_table_index, khm_replay_u32 num_active_tokens,
                                    khm_replay_u32 num_active_q_token_tiles, const uint32_t* replay_parameters, void* stream) {
+    return sliced_q_direct(compute, buffers, nullptr, page_table_index, num_active_tokens, num_active_q_token_tiles, replay_parameters, stream);
+}
+
+extern "C" int khm_sliced_q_direct_gated(const khm_sliced_q* compute, const khm_sliced_q_direct_buffers* buffers, khm_buffer gates,
+                                         khm_replay_u32 page_table_index, khm_replay_u32 num_active_tokens,
+                                         khm_replay_u32 num_active_q_token_tiles, const uint32_t* replay_parameters, void* stream) {
+    return sliced_q_direct(compute, buffers, &gates, page_table_index, num_active_tokens, num_active_q_token_tiles, replay_parameters, stream);
+}
+
+static int sliced_q_reduce(const khm_sliced_q* compute, const khm_sliced_q_reduce_buffers* buffers, const khm_buffer* gates,
+                           khm_replay_u32 num_active_q_token_tiles, const uint32_t* replay_parameters, void* stream) {
     clear_error();
     KHM_REQUIRE(compute != nullptr && buffers != nullptr, "compute and buffers must not be null");
     KHM_REQUIRE(!compute->direct, "GQA SplitKV SlicedQ direct-output compute has no Reduce");
@@ -762,6 +778,10 @@ extern "C" int khm_sliced_q_reduce(const khm_sliced_q* compute, const khm_sliced
     p.q_token_ranges = static_cast<const uint32_t*>(buffers->q_token_ranges.ptr);
     p.cu_partial_outputs = static_cast<const uint32_t*>(buffers->cu_sdpa_partial_outputs.ptr);
     p.gates = nullptr;
+    if (gates != nullptr) {
+        KHM_BUFFER_AT_LEAST(*gates, khm_gqa_sdpa_q_bytes(&config, &shape), "gates");
+        p.gates = static_cast<const uint16_t*>(gates->ptr);
+    }
     p.output = static_cast<uint16_t*>(buffers->output.ptr);
     p.replay_parameters = replay_parameters;
     p.num_active = to_device(num_active_q_token_tiles);
@@ -774,6 +794,16 @@ extern "C" int khm_sliced_q_reduce(const khm_sliced_q* compute, const khm_sliced
     launch_reduce_kernel(config, shape, true, shape.num_total_q_token_tiles, compute->variant.map_max_q_tokens, compute->reduce, p,
                          static_cast<hipStream_t>(stream));
     return check_launch("sliced-Q reduce");
+}
+
+extern "C" int khm_sliced_q_reduce(const khm_sliced_q* compute, const khm_sliced_q_reduce_buffers* buffers,
+                                   khm_replay_u32 num_active_q_token_tiles, const uint32_t* replay_parameters, void* stream) {
+    return sliced_q_reduce(compute, buffers, nullptr, num_active_q_token_tiles, replay_parameters, stream);
+}
+
+extern "C" int khm_sliced_q_reduce_gated(const khm_sliced_q* compute, const khm_sliced_q_reduce_buffers* buffers, khm_buffer gates,
+                                         khm_replay_u32 num_active_q_token_tiles, const uint32_t* replay_parameters, void* stream) {
+    return sliced_q_reduce(compute, buffers, &gates, num_active_q_token_tiles, replay_parameters, stream);
 }
 
 // ------------------------------------------------------------------------------------------ gate

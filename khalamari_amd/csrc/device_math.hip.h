@@ -121,6 +121,17 @@ __device__ __forceinline__ float sigmoid_bf16_steps(float x) {
     return x < 0.0f ? round_to_bf16(1.0f - y) : y;
 }
 
+// Four attention values times sigmoid(gate) as gqa_activation_gate_bf16 computes it from the bf16-rounded attention
+// output (gqa_activation_gate.metal:19-39); `gates` points at the four bf16 gate values of the same elements.
+__device__ __forceinline__ f32x4 gate_bf16x4(f32x4 attention, const uint16_t* gates) {
+    const uint2 gate_bits = *reinterpret_cast<const uint2*>(gates);
+    const float gate[4] = {bf16_bits_to_f32(gate_bits.x & 0xffffu), bf16_bits_to_f32(gate_bits.x >> 16),
+                           bf16_bits_to_f32(gate_bits.y & 0xffffu), bf16_bits_to_f32(gate_bits.y >> 16)};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) attention[i] = round_to_bf16(attention[i]) * sigmoid_bf16_steps(gate[i]);
+    return attention;
+}
+
 // gqa_activation_gate.metal:14-17.
 __device__ __forceinline__ float sigmoid_f32(float x) {
     const float y = 1.0f / (1.0f + __expf(-fabsf(x)));

@@ -50,7 +50,7 @@ struct MapParams {
     const uint32_t* cu_partial_outputs;  // [R + 1]
     uint32_t* arrival_counters;          // [R][gridDim.y], zero before the first launch; the merging block re-arms its counter
     uint16_t* final_output;              // bf16 [T][Hq][D]
-    const uint16_t* gates;               // bf16 [T][Hq][D] or nullptr
+    const uint16_t* gates;               // bf16 [T][Hq][D] or nullptr: gate of the fused Reduce, or of direct output
 };
 
 // Arguments of the flat (sliced-KV) and ranged (sliced-Q) Reduce kernels.

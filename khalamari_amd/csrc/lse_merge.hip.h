@@ -102,13 +102,7 @@ __device__ __forceinline__ MergeState merge_combine_slices(const float* stats, c
 __device__ __forceinline__ void merge_store_output(const MergeState& state, uint16_t* output, const uint16_t* gates, uint64_t out_index) {
     f32x4 result = {0.0f, 0.0f, 0.0f, 0.0f};
     if (state.run_sum > 0.0f) result = state.acc / state.run_sum;
-    if (gates != nullptr) {
-        const uint2 gate_bits = *reinterpret_cast<const uint2*>(gates + out_index);
-        const float gate[4] = {bf16_bits_to_f32(gate_bits.x & 0xffffu), bf16_bits_to_f32(gate_bits.x >> 16),
-                               bf16_bits_to_f32(gate_bits.y & 0xffffu), bf16_bits_to_f32(gate_bits.y >> 16)};
-#pragma unroll
-        for (int i = 0; i < 4; ++i) result[i] = round_to_bf16(result[i]) * sigmoid_bf16_steps(gate[i]);
-    }
+    if (gates != nullptr) result = gate_bf16x4(result, gates + out_index);
     const uint2 packed = make_uint2(pack_bf16x2(result[0], result[1]), pack_bf16x2(result[2], result[3]));
     *reinterpret_cast<uint2*>(output + out_index) = packed;
 }

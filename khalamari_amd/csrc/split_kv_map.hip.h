@@ -564,6 +564,7 @@ __global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapPara
                 *reinterpret_cast<f32x4*>(target) = value;
             }
         } else {
+            if (mode == kMapDirectBf16 && p.gates != nullptr) value = gate_bf16x4(value, p.gates + state * D + d);
             const uint2 packed = make_uint2(pack_bf16x2(value[0], value[1]), pack_bf16x2(value[2], value[3]));
             uint16_t* target = reinterpret_cast<uint16_t*>(p.out) + state * D + d;
             if (fused) {

@@ -915,8 +915,10 @@ void tile_map_kernel(const MapParams p) {
         }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            const f32x4 value = acc[nt][mt] * inverse;
+            f32x4 value = acc[nt][mt] * inverse;
             const uint32_t d = mt * 16 + g * 4;
+            // direct output of a gated layer: the sigmoid gate of the final bf16 value, as the Reduce applies it
+            if (mode == kMapDirectBf16 && p.gates != nullptr) value = gate_bf16x4(value, p.gates + row * D + d);
             if (mode == kMapPartialF32) {
                 *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.out) + row * D + d) = value;
             } else {

@@ -97,18 +97,28 @@ class Compute:
 
     def invoke_direct(self, *, q, kv_pages, req_slots, page_ids, visible_kv_token_ranges, q_token_ranges,
                       sdpa_map_task_templates, output, page_table_index: ReplayU32, num_active_tokens: ReplayU32,
-                      num_active_q_token_tiles: ReplayU32, replay_parameters=None, stream=None) -> None:
+                      num_active_q_token_tiles: ReplayU32, replay_parameters=None, stream=None, gates=None) -> None:
+        """`gates` (bf16 [T][Hq][D]) fuses the sigmoid gate that follows the SDPA into the output write."""
         buffers = SlicedQDirectBuffers(view(q), view(kv_pages), view(req_slots), view(page_ids),
                                        view(visible_kv_token_ranges), view(q_token_ranges),
                                        view(sdpa_map_task_templates), view(output))
+        if gates is not None:
+            _lib.check(_lib.lib().khm_sliced_q_direct_gated(self._handle, ctypes.byref(buffers), view(gates), page_table_index,
+                                                            num_active_tokens, num_active_q_token_tiles,
+                                                            param_block(replay_parameters), stream_handle(stream)))
+            return
         _lib.check(_lib.lib().khm_sliced_q_direct(self._handle, ctypes.byref(buffers), page_table_index,
                                                   num_active_tokens, num_active_q_token_tiles,
                                                   param_block(replay_parameters), stream_handle(stream)))
 
     def invoke_reduce(self, *, partial_output, partial_exp_sums, partial_max_logits, q_token_ranges,
                       cu_sdpa_partial_outputs, output, num_active_q_token_tiles: ReplayU32, replay_parameters=None,
-                      stream=None) -> None:
+                      stream=None, gates=None) -> None:
         buffers = SlicedQReduceBuffers(view(partial_output), view(partial_exp_sums), view(partial_max_logits),
                                        view(q_token_ranges), view(cu_sdpa_partial_outputs), view(output))
+        if gates is not None:
+            _lib.check(_lib.lib().khm_sliced_q_reduce_gated(self._handle, ctypes.byref(buffers), view(gates), num_active_q_token_tiles,
+                                                            param_block(replay_parameters), stream_handle(stream)))
+            return
         _lib.check(_lib.lib().khm_sliced_q_reduce(self._handle, ctypes.byref(buffers), num_active_q_token_tiles,
                                                   param_block(replay_parameters), stream_handle(stream)))

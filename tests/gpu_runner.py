@@ -69,8 +69,9 @@ def run_sliced_kv(w, templates, cu, device, *, max_q_heads=None, partial_dtype=D
 
 
 def run_sliced_q(w, ranges, templates, cu, device, *, kind, max_q_tokens, max_q_heads, stage=16, direct=False,
-                 partial_dtype=DTYPE_BF16, poison=0x4228, visible=None):
-    """Verify / prefill path: Map (or direct) over Q ranges, then the ranged Reduce.  Returns f32 [T, Hq, D]."""
+                 partial_dtype=DTYPE_BF16, poison=0x4228, visible=None, gates=None):
+    """Verify / prefill path: Map (or direct) over Q ranges, then the ranged Reduce; `gates` (bf16 bits [T, Hq, D]) fuses
+    the sigmoid gate into whichever of the two writes the output.  Returns f32 [T, Hq, D]."""
     g = w.geom
     config = component_config(w, sliced_q.Config, partial_dtype)
     variant = sdpa.ExecutionVariant.sliced_q(config.sdpa_config(), kind, max_q_tokens, stage, max_q_heads)
@@ -90,8 +91,9 @@ def run_sliced_q(w, ranges, templates, cu, device, *, kind, max_q_tokens, max_q_
                   sdpa_map_task_templates=tmpl, page_table_index=ReplayU32.fixed(w.layer),
                   num_active_tokens=ReplayU32.fixed(w.num_tokens),
                   num_active_q_token_tiles=ReplayU32.fixed(ranges.shape[0]))
+    gates_d = to_device(gates, device) if gates is not None else None
     if direct:
-        compute.invoke_direct(output=out, **common)
+        compute.invoke_direct(output=out, gates=gates_d, **common)
     else:
         partial = torch.zeros(config.partial_output_bytes(variant, shape), dtype=torch.uint8, device=device)
         sums = torch.zeros(config.partial_output_stats_bytes(variant, shape), dtype=torch.uint8, device=device)
@@ -101,6 +103,6 @@ def run_sliced_q(w, ranges, templates, cu, device, *, kind, max_q_tokens, max_q_
                            num_active_kv_splits=ReplayU32.fixed(templates.shape[0]), **common)
         compute.invoke_reduce(partial_output=partial, partial_exp_sums=sums, partial_max_logits=maxs, q_token_ranges=rng_d,
                               cu_sdpa_partial_outputs=cu_d, output=out,
-                              num_active_q_token_tiles=ReplayU32.fixed(ranges.shape[0]))
+                              num_active_q_token_tiles=ReplayU32.fixed(ranges.shape[0]), gates=gates_d)
     torch.cuda.synchronize()
     return bf16_tensor_to_f32(out)

@@ -267,6 +267,35 @@ def test_fused_gate_and_standalone_gate(device):
         assert np.all(got[active:] == 7.0)
 
 
+@pytest.mark.parametrize("hq,hkv,d,tile,heads", [(24, 4, 256, 32, 6), (24, 4, 256, 8, 6), (64, 8, 128, 32, 8), (8, 2, 128, 4, 4), (6, 2, 128, 4, 3)])
+def test_gate_fused_into_the_sliced_q_outputs(device, hq, hkv, d, tile, heads):
+    """The gated layer in prefill and verify: the sigmoid gate applied where the sliced-Q path writes its output - the
+    direct Map's epilogue, the ranged Reduce - must give, bit for bit, what the standalone gate kernel gives on the
+    ungated bf16 output (GQA::record runs the gate right after the SDPA: backend.rs:413-421,
+    gqa_activation_gate.metal:19-39).  Twelve- and eight-wave prefill tiles, verify tiles and the one-tile kernel."""
+    histories = [700, 33, 1500]
+    q_lens = [70, 5, 40] if tile >= 32 else [5, 2, 4]
+    w = helpers.make_workload(num_q_heads=hq, num_kv_heads=hkv, head_dim=d, tokens_per_page=16, histories=histories, q_lens=q_lens,
+                              seed=77 + tile)
+    rng = np.random.default_rng(78)
+    gate_bits = oracle.f32_to_bf16_bits((rng.standard_normal((w.num_tokens, hq, d)) * 2).astype(np.float32))
+    for kv_slice, direct in [(1 << 20, True), (256, False)]:
+        ranges, templates, cu = helpers.fixed_slice_plan(histories, q_lens, tile, kv_slice)
+        run = lambda gates: gpu_runner.run_sliced_q(w, ranges, templates, cu, device, kind=sdpa.MAP_Q_TOKENS_AND_HEADS,  # noqa: E731
+                                                    max_q_tokens=tile, max_q_heads=heads, stage=64, direct=direct, gates=gates)
+        print(f"gated sliced-Q hq={hq} d={d} tile={tile}x{heads} direct={direct}", flush=True)
+        plain, fused = run(None), run(gate_bits)
+        want = oracle.bf16_bits_to_f32(oracle.gate_bf16(oracle.f32_to_bf16_bits(plain), gate_bits))
+        assert np.array_equal(fused, want.reshape(fused.shape))
+        attn = gpu_runner.to_device(oracle.f32_to_bf16_bits(plain), device)
+        out = torch.zeros_like(attn)
+        activation_gate.invoke(DTYPE_BF16, hq, d, w.num_tokens, attn, gpu_runner.to_device(gate_bits, device), out, ReplayU32.fixed(w.num_tokens))
+        torch.cuda.synchronize()
+        assert np.array_equal(gpu_runner.bf16_tensor_to_f32(out).reshape(fused.shape), fused)
+    expected = oracle.gate_f32(helpers.expected_output(w), oracle.bf16_bits_to_f32(gate_bits))
+    helpers.assert_parity(fused, expected, "gated sliced-Q against the gated oracle", abs_tol=4e-3)
+
+
 def test_device_gate_matches_the_oracle_on_every_bf16_gate_value(device):
     """All 65 536 bf16 gate bit patterns, each against several attention values, bit for bit: the device evaluates the
     exponential with v_exp_f32, the oracle with libm, and every intermediate is rounded to bf16
