@@ -775,13 +775,12 @@ void tile_map_kernel(const MapParams p) {
             }
         }
     };
-    // Steady state of an interior run (direct loads, untracked weights): every tile of
+    // Steady state of an interior run (direct loads; weights untracked with every column anchored, or tracked): every tile of
     // [tile_begin, tile_end) has its successor's first slice in the range, and the tile NSTAGES - 1 ahead exists and lies
     // wholly inside the block's KV range.  One straight-line body per tile: a fixed wait, the barrier, unconditional
     // requests; the compiler is free to mix the S^T of the next slice with the softmax of this one.
-    auto run_steady_tiles = [&](uint32_t tile_begin, uint32_t tile_end) __attribute__((always_inline)) {
+    auto run_steady_tiles = [&](auto untracked_anchored, uint32_t tile_begin, uint32_t tile_end) __attribute__((always_inline)) {
         constexpr std::false_type no{};
-        constexpr std::integral_constant<int, 2> untracked_anchored{};
         TileIds ahead = fetch_ids_interior(tile_begin + NSTAGES - 1);
         for (uint32_t tile = tile_begin; tile < tile_end; ++tile) {
             wait_vmem_outstanding<(NSTAGES - 3) * LPW>();   // tile + 1 has landed; tiles up to tile + NSTAGES - 2 are requested
@@ -860,33 +859,37 @@ void tile_map_kernel(const MapParams p) {
             run_tiles(yes, yes, no, tail_begin, num_tiles);
         } else {
             run_tiles(no, yes, no, 0, head_end);
+            // tiles t with t + NSTAGES - 1 a whole tile inside [blk_lo, blk_hi), (t + NSTAGES) * BK <= blk_hi - first_token, run in
+            // the steady-state loop
+            uint32_t steady_limit = head_end;
+            if constexpr (!STAGED8) {
+                const uint32_t whole_tiles = (blk_hi - first_token) / BK;
+                steady_limit = whole_tiles >= (uint32_t)NSTAGES ? whole_tiles - (NSTAGES - 1) : 0;
+                steady_limit = steady_limit < tail_begin ? steady_limit : tail_begin;
+                steady_limit = steady_limit > head_end ? steady_limit : head_end;
+            }
             if constexpr (DIRECT) {
                 // no partial state to hand on: the interior slices need not follow the largest score
 #pragma unroll
                 for (int nt = 0; nt < NTW; ++nt) unanchored = unanchored | (lane_top[nt] == -INFINITY);
-                uint32_t steady_end = head_end;
-                if constexpr (!STAGED8) {
-                    // tiles t with t + NSTAGES - 1 a whole tile inside [blk_lo, blk_hi): (t + NSTAGES) * BK <= blk_hi - first_token
-                    const uint32_t whole_tiles = (blk_hi - first_token) / BK;
-                    uint32_t limit = whole_tiles >= (uint32_t)NSTAGES ? whole_tiles - (NSTAGES - 1) : 0;
-                    limit = limit < tail_begin ? limit : tail_begin;
-                    if (limit > head_end) {
-                        uint32_t steady_begin = head_end;
-                        if (__builtin_amdgcn_ballot_w64(unanchored) != 0) {
-                            // a column without a reference yet: the general slice anchors it
-                            run_tiles(no, no, yes, head_end, head_end + 1);
-                            steady_begin = head_end + 1;
-                        }
-                        steady_end = limit;
-                        if (steady_end > steady_begin) {
-                            run_steady_tiles(steady_begin, steady_end);
-                            upcoming = fetch_ids(steady_end + NSTAGES - 1);
-                        }
-                    }
+                uint32_t steady_begin = head_end;
+                if (steady_limit > head_end && __builtin_amdgcn_ballot_w64(unanchored) != 0) {
+                    // a column without a reference yet: the general slice anchors it
+                    run_tiles(no, no, yes, head_end, head_end + 1);
+                    steady_begin = head_end + 1;
                 }
-                run_tiles(no, no, yes, steady_end, tail_begin);
+                if (steady_limit > steady_begin) {
+                    run_steady_tiles(std::integral_constant<int, 2>{}, steady_begin, steady_limit);
+                    upcoming = fetch_ids(steady_limit + NSTAGES - 1);
+                    steady_begin = steady_limit;
+                }
+                run_tiles(no, no, yes, steady_begin, tail_begin);
             } else {
-                run_tiles(no, no, no, head_end, tail_begin);
+                if (steady_limit > head_end) {
+                    run_steady_tiles(no, head_end, steady_limit);
+                    upcoming = fetch_ids(steady_limit + NSTAGES - 1);
+                }
+                run_tiles(no, no, no, steady_limit, tail_begin);
             }
             run_tiles(no, yes, no, tail_begin, num_tiles);
         }
