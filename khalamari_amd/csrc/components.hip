@@ -48,8 +48,12 @@ static TileKernelChoice select_tile_kernel(uint32_t head_dim, uint32_t coordinat
     // column-tile kernels at D 128 and the eight-wave tile at D 256 (523 -> 638 TFLOP/s on 2048-token chunks at
     // Hq24/Hkv4); the bandwidth-bound verify tiles have nothing to gain.
     // Twelve waves of one column tile each for 129..192 coordinates at D 256 (32 tokens x 6 Q heads of a KV head: no idle
-    // column, three waves per SIMD); bf16 pages only, FP8 pages keep the 256-column build for such tiles.
-    if (head_dim == 256 && coordinates > 128 && coordinates <= 192 && kv_dtype != KHM_DTYPE_FP8_E4M3FN) {
+    // column, three waves per SIMD), on bf16 and on FP8 pages.
+    if (head_dim == 256 && coordinates > 128 && coordinates <= 192) {
+        if (kv_dtype == KHM_DTYPE_FP8_E4M3FN) {
+            if (direct) return {tile_map_kernel<256, 1, 12, 32, 4, 1, true, true>, 768, (uint32_t)TileSmem<256, 32, 4>::kBytes};
+            return {tile_map_kernel<256, 1, 12, 32, 4, 1, true>, 768, (uint32_t)TileSmem<256, 32, 4>::kBytes};
+        }
         if (direct) return {tile_map_kernel<256, 1, 12, 32, 4, 1, false, true>, 768, (uint32_t)TileSmem<256, 32, 4, 512, true>::kBytes};
         return {tile_map_kernel<256, 1, 12, 32, 4, 1>, 768, (uint32_t)TileSmem<256, 32, 4, 512, true>::kBytes};
     }

@@ -107,18 +107,24 @@ void tile_map_kernel(const MapParams p) {
     constexpr int PAGE_ROW = D * (KV8 ? 1 : 2);     // bytes of one K/V row in a page
     constexpr int CPR = PAGE_ROW / 16;              // 16-byte chunks per K/V row in a page
     constexpr bool LINEAR = tile_layout_is_linear(D, KV8);
-    constexpr int HALVES = LINEAR ? D / 128 : 1;    // linear layout: wave loads per row group (each takes 128 dims of four rows)
-    constexpr int RPL = LINEAR ? 4 : 64 / CPR;      // rows per wave load
+    constexpr bool LINEAR_LOADS = LINEAR && !KV8;   // direct-to-LDS loads that fill the linear layout's units themselves
+    constexpr int HALVES = LINEAR_LOADS ? D / 128 : 1;    // ... wave loads per row group (each takes 128 dims of four rows)
+    constexpr int RPL = LINEAR_LOADS ? 4 : 64 / CPR;      // rows per wave load
     constexpr int UNITS = BK * CPR / 64;            // wave loads per plane and tile
     // PAIRED: the units divide evenly over the waves; a wave then loads K and V of the same units, which share their page
     // id and scalar base.  Otherwise (twelve waves over sixteen units) the 2 * UNITS loads of a tile are dealt out as one
     // list, two or three to a wave, and a wave with fewer repeats its last one so that every wave counts the same number
     // of loads per tile (the waits are compile-time constants).
-    constexpr bool PAIRED = UNITS % NWAVES == 0;
-    constexpr int UPW = PAIRED ? UNITS / NWAVES : 1;                           // units per wave (paired form)
+    // FP8 tiles staged through registers have half as many units; when there are fewer than waves (twelve waves over
+    // eight units) the first UNITS waves load one unit each and the others none (those loads are ordinary ones the
+    // compiler waits for, so nothing has to be counted).
+    constexpr int LOADERS = (KV8 && UNITS < NWAVES) ? UNITS : NWAVES;          // waves that load
+    constexpr bool PAIRED = UNITS % LOADERS == 0;
+    constexpr int UPW = PAIRED ? UNITS / LOADERS : 1;                          // units per loading wave (paired form)
     constexpr int LPW = PAIRED ? 2 * UPW : (2 * UNITS + NWAVES - 1) / NWAVES;  // loads per wave and tile
     constexpr int IDS = PAIRED ? UPW : LPW;                                    // page ids per wave and tile
     static_assert(PAIRED || !KV8, "FP8 tiles are written for evenly divided units");
+    static_assert(LOADERS == NWAVES || (KV8 && !(NTW == 1 && NWAVES == 4)), "only register-staged FP8 tiles leave waves without loads");
     static_assert((SL == 1 || SL == 2) && NSTAGES >= 3 && NSTAGES <= 5, "unsupported tiling");
     constexpr bool RAW8 = KV8 && NTW == 1 && NWAVES == 4;   // raw FP8 codes in LDS, decoded by the waves that read them
     constexpr bool STAGED8 = KV8 && !RAW8;       // FP8 tiles decoded once on their way into bf16 LDS tiles
@@ -134,7 +140,7 @@ void tile_map_kernel(const MapParams p) {
     // Where chunk `chunk` (16 bytes) of tile row `row` sits inside its K or V tile in LDS.
     // Unit n of a tile (the n-th wave load of a plane): its first row, and its place among the tile's units in LDS.
     auto unit_first_row = [](uint32_t n) -> uint32_t { return (n / HALVES) * RPL; };
-    auto unit_position = [](uint32_t n) -> uint32_t { return LINEAR ? (n % HALVES) * (BK / 4) + n / HALVES : n; };
+    auto unit_position = [](uint32_t n) -> uint32_t { return LINEAR_LOADS ? (n % HALVES) * (BK / 4) + n / HALVES : n; };
     auto k_place = [&](uint32_t row, uint32_t chunk) -> uint32_t {
         if constexpr (LINEAR) return ((chunk >> 4) * (BK / 4) + (row >> 2)) * 1024 + ((chunk >> 2) & 3u) * 256 + ((row & 3u) << 6) + ((((0u - chunk) ^ (row >> 2)) & 3u) << 4);
         else return row * ROW + ((chunk ^ k_swizzle_of(row)) << 4);
@@ -420,7 +426,9 @@ void tile_map_kernel(const MapParams p) {
     // FP8 pages: one tile in registers, decoded into the bf16 LDS layout the direct loads would have produced
     // (source chunk c of a K row lands at position c ^ (row & 15), of a V row at c ^ 2 (row & 7)).
     uint4 raw_k[STAGED8 ? UPW : 1], raw_v[STAGED8 ? UPW : 1];
+    const bool loads_raw_tiles = LOADERS == NWAVES || wave < LOADERS;   // wave-uniform
     auto load_raw_tile = [&](uint32_t tile, const TileIds ids) __attribute__((always_inline)) {
+        if (!loads_raw_tiles) return;
         const uint32_t load_row = lane / CPR;
         const uint32_t load_pos = lane % CPR;
         const uint32_t tile_token = first_token + tile * BK;
@@ -435,7 +443,24 @@ void tile_map_kernel(const MapParams p) {
             raw_v[i] = *reinterpret_cast<const uint4*>(page + plane_v + offset);
         }
     };
+    // the same for a tile wholly inside [blk_lo, blk_hi): no clamps, lane offsets that do not depend on the tile
+    uint32_t raw_lane_offset[STAGED8 ? UPW : 1];
+    if constexpr (STAGED8) {
+#pragma unroll
+        for (int i = 0; i < UPW; ++i)
+            raw_lane_offset[i] = ((first_token + (wave * UPW + i) * RPL + lane / CPR) & (tpp - 1)) * PAGE_ROW + (lane % CPR) * 16;
+    }
+    auto load_raw_tile_interior = [&](const TileIds ids) __attribute__((always_inline)) {
+        if (!loads_raw_tiles) return;
+#pragma unroll
+        for (int i = 0; i < UPW; ++i) {
+            const unsigned char* page = k_plane_base + (uint64_t)ids[i] * p.page_bytes;
+            raw_k[i] = *reinterpret_cast<const uint4*>(page + raw_lane_offset[i]);
+            raw_v[i] = *reinterpret_cast<const uint4*>(page + (plane_v - plane_k) + raw_lane_offset[i]);
+        }
+    };
     auto write_raw_tile = [&](uint32_t tile) __attribute__((always_inline)) {
+        if (!loads_raw_tiles) return;
         const uint32_t load_row = lane / CPR;
         const uint32_t load_pos = lane % CPR;
         unsigned char* k_stage = k_lds + (tile % NSTAGES) * Smem::kKTileBytes;
@@ -783,13 +808,20 @@ void tile_map_kernel(const MapParams p) {
         constexpr std::false_type no{};
         TileIds ahead = fetch_ids_interior(tile_begin + NSTAGES - 1);
         for (uint32_t tile = tile_begin; tile < tile_end; ++tile) {
-            wait_vmem_outstanding<(NSTAGES - 3) * LPW>();   // tile + 1 has landed; tiles up to tile + NSTAGES - 2 are requested
+            // direct loads: tile + 1 has landed, tiles up to tile + NSTAGES - 2 are requested; FP8 tiles staged through
+            // registers: tile + 1 is in LDS, tile + 2 in registers, tile + 3 is requested here (the compiler waits for it)
+            if constexpr (!STAGED8) wait_vmem_outstanding<(NSTAGES - 3) * LPW>();
             barrier_keeping_loads_in_flight();
             const uint32_t stage = tile % NSTAGES, next_stage = (tile + 1) % NSTAGES, free_stage = (tile + NSTAGES - 1) % NSTAGES;
             const unsigned char* k_tile = k_lds + stage * Smem::kKTileBytes;
             const unsigned char* v_tile = v_lds + stage * Smem::kVTileBytes;
             auto request_next = [&]() __attribute__((always_inline)) {
-                issue_interior_tile(free_stage, ahead);
+                if constexpr (STAGED8) {
+                    write_raw_tile(tile + 2);
+                    load_raw_tile_interior(ahead);
+                } else {
+                    issue_interior_tile(free_stage, ahead);
+                }
                 ahead = fetch_ids_interior(tile + NSTAGES);
             };
             auto nothing = []() __attribute__((always_inline)) {};
@@ -862,7 +894,7 @@ void tile_map_kernel(const MapParams p) {
             // tiles t with t + NSTAGES - 1 a whole tile inside [blk_lo, blk_hi), (t + NSTAGES) * BK <= blk_hi - first_token, run in
             // the steady-state loop
             uint32_t steady_limit = head_end;
-            if constexpr (!STAGED8) {
+            {
                 const uint32_t whole_tiles = (blk_hi - first_token) / BK;
                 steady_limit = whole_tiles >= (uint32_t)NSTAGES ? whole_tiles - (NSTAGES - 1) : 0;
                 steady_limit = steady_limit < tail_begin ? steady_limit : tail_begin;

@@ -59,7 +59,8 @@ def test_fp8_spec_verify_blocks(device):
         helpers.assert_parity(actual, expected, "fp8 verify")
 
 
-@pytest.mark.parametrize("hq,hkv,d,tile", [(64, 8, 128, 32), (32, 4, 128, 16), (24, 4, 256, 16), (16, 2, 256, 32)])
+@pytest.mark.parametrize("hq,hkv,d,tile", [(64, 8, 128, 32), (32, 4, 128, 16), (24, 4, 256, 16), (16, 2, 256, 32), (24, 4, 256, 32),
+                                           (12, 2, 256, 32)])
 def test_fp8_chunked_prefill_onto_a_paged_prefix(device, hq, hkv, d, tile):
     """Causal chunks appended to paged prefixes on FP8 pages: wide Q tiles on the LDS-tiled kernel, whose tiles are
     decoded on their way into LDS; direct output and split-KV + Reduce; the FP8 NaN code in every unused page slot."""
@@ -74,6 +75,21 @@ def test_fp8_chunked_prefill_onto_a_paged_prefix(device, hq, hkv, d, tile):
         actual = gpu_runner.run_sliced_q(w, ranges, templates, cu, device, kind=sdpa.MAP_Q_TOKENS_AND_HEADS, max_q_tokens=tile,
                                          max_q_heads=hq // hkv, stage=64, direct=direct)
         helpers.assert_parity(actual, expected, f"fp8 prefill tile={tile} slice={kv_slice} direct={direct}")
+
+
+def test_fp8_long_interior_runs_of_the_twelve_wave_tile_checked_on_every_row(device):
+    """Hq12/Hkv2/D256 (six Q heads per KV head, 32-token tiles: 192 columns on twelve waves) over FP8 pages with prefixes of
+    a few thousand keys, so that the steady-state loop of the register-staged FP8 tiles carries nearly every tile."""
+    histories, q_lens = [3000, 1531], [70, 40]
+    w = helpers.make_workload(num_q_heads=12, num_kv_heads=2, head_dim=256, tokens_per_page=16, histories=histories, q_lens=q_lens,
+                              seed=611, garbage_bits=0x7F, fp8_pages=True)
+    expected = helpers.expected_output(w)
+    for kv_slice, direct in [(1 << 20, True), (1024, False)]:
+        ranges, templates, cu = helpers.fixed_slice_plan(histories, q_lens, 32, kv_slice)
+        print(f"fp8 twelve-wave tile kv_slice={kv_slice} direct={direct}", flush=True)
+        actual = gpu_runner.run_sliced_q(w, ranges, templates, cu, device, kind=sdpa.MAP_Q_TOKENS_AND_HEADS, max_q_tokens=32, max_q_heads=6,
+                                         stage=64, direct=direct)
+        helpers.assert_parity(actual, expected, f"fp8 twelve-wave tile slice={kv_slice} direct={direct}")
 
 
 @pytest.mark.parametrize("tpp", [8, 32])

@@ -75,7 +75,8 @@ def test_decode_configs_at_full_size(device, index, fp8):
     helpers.record_parity(f"config{index}{'_fp8_pages' if fp8 else ''} full size, bf16 output, {len(tokens)} tokens", stats)
 
 
-@pytest.mark.parametrize("index,fp8", [(4, False), (4, True), (5, False), (5, True), (bench.EXTRA_PREFILL_D256, False)])
+@pytest.mark.parametrize("index,fp8", [(4, False), (4, True), (5, False), (5, True), (bench.EXTRA_PREFILL_D256, False),
+                                       (bench.EXTRA_PREFILL_D256, True)])
 def test_verify_and_prefill_configs_at_full_size(device, index, fp8):
     workload = bench.Workload(index, device, num_pools=1, fp8_pages=fp8)
     actual = _run_step(workload)

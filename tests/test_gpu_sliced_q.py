@@ -426,7 +426,7 @@ def test_long_interior_runs_of_a_prefill_tile_checked_on_every_row(device, hq, h
 
 @pytest.mark.parametrize("hq,hkv,d,tile,fp8", [(64, 8, 128, 32, False), (64, 8, 128, 16, False), (64, 8, 128, 32, True),
                                                (32, 4, 128, 16, True), (32, 8, 128, 4, False), (24, 4, 256, 16, False),
-                                               (24, 4, 256, 16, True), (24, 4, 256, 32, False)])
+                                               (24, 4, 256, 16, True), (24, 4, 256, 32, False), (24, 4, 256, 32, True)])
 def test_scores_that_keep_outgrowing_the_running_reference(device, hq, hkv, d, tile, fp8):
     """Every score of a sequence rises steadily along the context (by some 60 octaves over 3000 keys), so later scores
     exceed the earlier maximum by far more than any rescaling threshold, over and over: the reference-moving path of
