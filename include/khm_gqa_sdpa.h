@@ -434,7 +434,9 @@ typedef struct khm_bidi_block_sdpa_buffers {
     khm_buffer partial_output;
 } khm_bidi_block_sdpa_buffers;
 /* Compute::invoke + Invocation::record (bidi_block_sdpa.rs:227-287): one launch, enqueued on `stream`.  A Fixed
- * num_active_q_token_ranges must equal num_total_q_token_ranges, as in the reference (bidi_block_sdpa.rs:292-294). */
+ * num_active_q_token_ranges must equal num_total_q_token_ranges, as in the reference (bidi_block_sdpa.rs:292-294).
+ * head_dim must be a multiple of 32 and at most 1024 (KHM_ERR_UNSUPPORTED beyond: a lane holds at most eight
+ * 8-element chunks of a Q row); the reference's Config::validate has no upper bound. */
 int khm_bidi_block_sdpa(const khm_bidi_block_sdpa_config* config, const khm_bidi_block_sdpa_shape* shape,
                         const khm_bidi_block_sdpa_buffers* buffers, khm_replay_u32 num_active_q_token_ranges,
                         const uint32_t* replay_parameters, void* stream);

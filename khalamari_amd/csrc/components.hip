@@ -5,6 +5,8 @@
 // (.../gqa/activation_gate.rs:35-168).  Nothing here allocates or synchronizes.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "common.h"
 #include "device_params.h"
 #include "reduce_gate.hip.h"
@@ -323,7 +325,10 @@ extern "C" int khm_sliced_kv_create(const khm_gqa_sdpa_config* config, const khm
     // Set-up is the place to look up this device's copy of the static scratch array (khm_sliced_kv_map_reduce_static),
     // so that the entry point itself makes no runtime query on its first call.  Failing here is not an error of create.
     unsigned char* static_scratch = nullptr;
-    if (static_scratch_pointer(&static_scratch) != KHM_OK) clear_error();
+    if (static_scratch_pointer(&static_scratch) != KHM_OK) {
+        clear_error();
+        (void)hipGetLastError();   // the failed query must not show up as the next launch's error
+    }
     *out = compute;
     return KHM_OK;
 }
@@ -438,7 +443,7 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 constexpr int kMaxDevices = 64;
 // filled when a compute is created on a device (else on the entry point's first call there); concurrent fills store the same value
-static unsigned char* static_scratch_of_device[kMaxDevices];
+static std::atomic<unsigned char*> static_scratch_of_device[kMaxDevices];
 
 __global__ __launch_bounds__(256) void clear_u32_kernel(uint32_t* words, uint32_t count) {
     const uint32_t index = blockIdx.x * 256 + threadIdx.x;
@@ -450,14 +455,16 @@ static int static_scratch_pointer(unsigned char** out) {
     hipError_t status = hipGetDevice(&device);
     if (status != hipSuccess) return fail(KHM_ERR_HIP, "hipGetDevice failed: %s", hipGetErrorString(status));
     KHM_REQUIRE(device >= 0 && device < kMaxDevices, "device index %d is outside the static scratch table", device);
-    if (static_scratch_of_device[device] == nullptr) {
+    unsigned char* known = static_scratch_of_device[device].load(std::memory_order_acquire);
+    if (known == nullptr) {
         void* address = nullptr;
         status = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
         if (status != hipSuccess || address == nullptr)
             return fail(KHM_ERR_HIP, "hipGetSymbolAddress(scratch) failed on device %d: %s", device, hipGetErrorString(status));
-        static_scratch_of_device[device] = static_cast<unsigned char*>(address);
+        known = static_cast<unsigned char*>(address);
+        static_scratch_of_device[device].store(known, std::memory_order_release);
     }
-    *out = static_scratch_of_device[device];
+    *out = known;
     return KHM_OK;
 }
 

@@ -47,7 +47,8 @@ def test_fp8_unaligned_slices_and_nan_garbage(device):
 
 
 def test_fp8_spec_verify_blocks(device):
-    """q_len 2..5 causal blocks over FP8 pages: sliced-Q tiles of up to 64 coordinates run on the split-KV kernel."""
+    """q_len 2..5 causal blocks over FP8 pages: sliced-Q tiles of 17..64 coordinates run on the LDS-tiled kernel that keeps
+    the raw FP8 codes in LDS and decodes the fragments it reads."""
     histories, q_lens = [300, 17, 1000, 64], [2, 5, 3, 4]
     w = helpers.make_workload(num_q_heads=32, num_kv_heads=4, head_dim=128, tokens_per_page=16, histories=histories, q_lens=q_lens,
                               seed=33, fp8_pages=True)
@@ -57,6 +58,22 @@ def test_fp8_spec_verify_blocks(device):
         actual = gpu_runner.run_sliced_q(w, ranges, templates, cu, device, kind=sdpa.MAP_Q_TOKENS_AND_HEADS, max_q_tokens=8, max_q_heads=8,
                                          direct=direct)
         helpers.assert_parity(actual, expected, "fp8 verify")
+
+
+@pytest.mark.parametrize("tpp", [8, 16, 32])
+def test_fp8_spec_verify_blocks_at_head_dim_256(device, tpp):
+    """The same blocks at head dim 256 (Hq16/Hkv2, tiles of 8 tokens x 8 heads = 64 coordinates): raw rows of 256 bytes in
+    LDS, swizzled by row & 15 on both planes; split into 256- and 100-token slices + Reduce, and unsplit with direct output."""
+    histories, q_lens = [300, 17, 1000, 64], [2, 5, 3, 4]
+    w = helpers.make_workload(num_q_heads=16, num_kv_heads=2, head_dim=256, tokens_per_page=tpp, histories=histories, q_lens=q_lens,
+                              seed=35 + tpp, fp8_pages=True, garbage_bits=0x7F)
+    expected = helpers.expected_output(w)
+    for kv_slice, direct in [(256, False), (100, False), (1 << 20, True)]:
+        ranges, templates, cu = helpers.fixed_slice_plan(histories, q_lens, 8, kv_slice)
+        print(f"fp8 verify d=256 tpp={tpp} kv_slice={kv_slice} direct={direct}", flush=True)
+        actual = gpu_runner.run_sliced_q(w, ranges, templates, cu, device, kind=sdpa.MAP_Q_TOKENS_AND_HEADS, max_q_tokens=8, max_q_heads=8,
+                                         direct=direct)
+        helpers.assert_parity(actual, expected, f"fp8 verify d=256 tpp={tpp} slice={kv_slice} direct={direct}")
 
 
 @pytest.mark.parametrize("hq,hkv,d,tile", [(64, 8, 128, 32), (32, 4, 128, 16), (24, 4, 256, 16), (16, 2, 256, 32), (24, 4, 256, 32),

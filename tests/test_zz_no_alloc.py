@@ -82,3 +82,47 @@ def test_static_scratch_rejects_shapes_beyond_the_array(device):
                                          cu_sdpa_partial_outputs=small, output=dummy, page_table_index=ReplayU32.fixed(0),
                                          num_active_tokens=ReplayU32.fixed(64), num_active_kv_splits=ReplayU32.fixed(1024))
     torch.cuda.synchronize()
+
+
+def test_static_scratch_call_under_graph_capture_allocates_nothing(device):
+    """The claims the entry point exists for: it can be recorded into a HIP graph (stream capture forbids allocation, so a
+    hidden hipMalloc would fail the capture), device memory in use does not change across the call, and every replay -
+    with eager work and synchronizations in between - equals the eager result."""
+    histories = [1200, 300, 2047, 64]
+    q_lens = [1] * len(histories)
+    w = helpers.make_workload(num_q_heads=32, num_kv_heads=8, head_dim=128, tokens_per_page=16, histories=histories, q_lens=q_lens, seed=940)
+    _, templates, cu = helpers.fixed_slice_plan(histories, q_lens, 1, 256)
+    templates = np.asarray(templates, dtype=np.uint32).reshape(-1, 3)
+    g = w.geom
+    config = gpu_runner.component_config(w, sliced_kv.Config, DTYPE_BF16)
+    variant = sdpa.ExecutionVariant.sliced_kv(config.sdpa_config(), g.head_dim, 128, 4)
+    compute = sliced_kv.Compute(config, variant, sliced_kv.Shape(w.num_tokens, templates.shape[0]))
+    common = dict(q=gpu_runner.to_device(w.q_bits, device), kv_pages=gpu_runner.to_device(w.kv_pages, device),
+                  req_slots=gpu_runner.to_device(w.req_slots, device), page_ids=gpu_runner.to_device(w.page_ids, device),
+                  sdpa_map_task_templates=gpu_runner.to_device(templates, device),
+                  cu_sdpa_partial_outputs=gpu_runner.to_device(np.asarray(cu, dtype=np.uint32), device),
+                  page_table_index=ReplayU32.fixed(w.layer), num_active_tokens=ReplayU32.fixed(w.num_tokens),
+                  num_active_kv_splits=ReplayU32.fixed(templates.shape[0]))
+    out = torch.full((w.num_tokens, g.num_q_heads, g.head_dim), 0x4228, dtype=torch.int16, device=device)
+    compute.invoke_map_reduce_static(output=out, **common)      # eager: the reference result, and the warm-up before capture
+    torch.cuda.synchronize()
+    eager = out.cpu().numpy().copy()
+    helpers.assert_parity(oracle.bf16_bits_to_f32(eager.view(np.uint16)), helpers.expected_output(w), "static scratch, eager")
+
+    free_before, _ = torch.cuda.mem_get_info(device)
+    allocated_before = torch.cuda.memory_allocated(device)
+    compute.invoke_map_reduce_static(output=out, **common)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info(device)
+    assert free_after == free_before and torch.cuda.memory_allocated(device) == allocated_before
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        compute.invoke_map_reduce_static(output=out, **common)
+    for replay in range(3):
+        print(f"static scratch graph replay {replay}", flush=True)
+        out.fill_(0x4228)           # eager fill kernel between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), eager), f"replay {replay} differs from the eager call"
