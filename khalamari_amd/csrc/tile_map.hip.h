@@ -317,16 +317,19 @@ void tile_map_kernel(const MapParams p) {
     }
 
     // The Q loads have to be complete, in the compiler's eyes too, before the tile loop starts: a wait the compiler
-    // placed inside the loop would also drain the direct-to-LDS loads in flight, of which it knows nothing.
+    // placed inside the loop would also drain the direct-to-LDS loads in flight, of which it knows nothing.  The wait is
+    // placed behind the requests of the first tiles (see below), so that both round trips to memory run side by side.
+    auto settle_q_fragments = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int nt = 0; nt < NTW; ++nt)
+        for (int nt = 0; nt < NTW; ++nt)
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
-            U32x4 bits = __builtin_bit_cast(U32x4, q_frag[nt][ks]);
-            asm volatile("" : "+v"(bits));
-            q_frag[nt][ks] = __builtin_bit_cast(uint4, bits);
-        }
+            for (int ks = 0; ks < KS; ++ks) {
+                typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
+                U32x4 bits = __builtin_bit_cast(U32x4, q_frag[nt][ks]);
+                asm volatile("" : "+v"(bits));
+                q_frag[nt][ks] = __builtin_bit_cast(uint4, bits);
+            }
+    };
 
     // ---- tile schedule -------------------------------------------------------------------------------------
     const uint32_t first_group = blk_lo >> 4;                                   // 16-token groups
@@ -845,10 +848,12 @@ void tile_map_kernel(const MapParams p) {
                 write_raw_tile(1);
             }
             if (num_tiles > 2) load_raw_tile(2, fetch_ids(2));
+            settle_q_fragments();
         } else {
 #pragma unroll
             for (int t = 0; t < NSTAGES - 1; ++t)
                 if ((uint32_t)t < num_tiles) issue_tile(t, fetch_ids(t));
+            settle_q_fragments();
             // publish tile 0 and start the pipeline with the scores of the first slice
             wait_for_tile(0);
         }
