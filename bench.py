@@ -31,7 +31,7 @@ NUM_POOLS = 3
 # HBM bytes per Map launch from the hardware counters, (FETCH_SIZE * 2.000 + WRITE_SIZE * 1.000) KiB per dispatch:
 # two `rocprofv3 --pmc` runs per config, each counter scaled by what it reads for a plain 1 GiB copy kernel
 # (`--calibration-copy`).  The summaries with their commands are the text files under profiles/.
-MEASURED_MAP_TRAFFIC_BYTES = {2: 564_421_474, 3: 2_151_670_207, 4: 1_447_022_364, 5: 1_201_929_056}
+MEASURED_MAP_TRAFFIC_BYTES = {2: 564_443_136, 3: 2_151_780_352, 4: 1_447_216_128, 5: 1_202_862_080, 6: 1_068_921_856}
 
 CONFIGS = {
     1: dict(name="config1: B=1 q=1 Hq32/Hkv8/D128 ctx 1024, identity pages", hq=32, hkv=8, d=128, kind="decode", kv_slice=64),
@@ -55,10 +55,10 @@ SLAB_BYTES = 4096
 _slab_reader_lib = None
 
 
-def slab_read(pool, slab_ids, num_slabs: int, sink, blocks_per_cu: int = 2, run_slabs: int = 1) -> None:
-    """Enqueues, on torch's current stream, a launch that only reads `num_slabs` slabs of 4096 bytes of `pool` from a
-    resident grid, in the Map kernel's lane layout: slab i at byte offset `slab_ids[i] * 4096`, or with `run_slabs` > 1
-    runs of that many consecutive slabs, run j at `slab_ids[j] * run_slabs * 4096`.  The kernel lives in
+def slab_read(pool, slab_ids, num_slabs: int, sink, blocks_per_cu: int = 2, run_slabs: int = 1, slab_bytes: int = SLAB_BYTES) -> None:
+    """Enqueues, on torch's current stream, a launch that only reads `num_slabs` slabs of `slab_bytes` (4096 or 2048)
+    bytes of `pool` from a resident grid, in the Map kernel's lane layout: slab i at byte offset `slab_ids[i] * slab_bytes`,
+    or with `run_slabs` > 1 runs of that many consecutive slabs, run j at `slab_ids[j] * run_slabs * slab_bytes`.  The kernel lives in
     `libbench_slab_read.so` beside this file (source `bench_slab_read.hip`): a measurement aid, not part of the library."""
     import ctypes
 
@@ -68,7 +68,7 @@ def slab_read(pool, slab_ids, num_slabs: int, sink, blocks_per_cu: int = 2, run_
         return t.numel() * t.element_size()
 
     status = _bench_aid_lib().bench_slab_read(pool.data_ptr(), nbytes(pool), slab_ids.data_ptr(), nbytes(slab_ids), int(num_slabs),
-                                              int(run_slabs), int(blocks_per_cu), sink.data_ptr(), nbytes(sink),
+                                              int(run_slabs), int(slab_bytes), int(blocks_per_cu), sink.data_ptr(), nbytes(sink),
                                               ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
     if status != 0:
         raise RuntimeError(f"bench_slab_read failed with status {status}")
@@ -85,7 +85,8 @@ def _bench_aid_lib():
         _slab_reader_lib = ctypes.CDLL(path)
         _slab_reader_lib.bench_slab_read.restype = ctypes.c_int
         _slab_reader_lib.bench_slab_read.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint32,
-                                                     ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
+                                                     ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_uint64,
+                                                     ctypes.c_void_p]
     return _slab_reader_lib
 
 
@@ -341,33 +342,36 @@ class Workload:
 
     def slab_reader(self, steps: int) -> dict:
         """The memory system's own figure for this launch: a kernel that only reads as many bytes as the workload's
-        visible K/V, as 4 KB slabs at random places of the same pools (rotated like the steps), from a resident grid
+        visible K/V, as slabs (4 KB; 2 KB on FP8 pages at head_dim 128: what one page holds contiguously for one plane and
+        KV head) at random places of the same pools (rotated like the steps), from a resident grid
         with every wave the same share.  No metadata chain, no softmax, no merge, no ragged tail."""
         import torch
 
         spec = self.spec
         kv_bytes = self.visible_tokens * spec["hkv"] * spec["d"] * 2 * self.kv_element_bytes
-        pool_slabs = self.kv_pools[0].numel() * self.kv_pools[0].element_size() // SLAB_BYTES
-        num_slabs = min(kv_bytes // SLAB_BYTES, pool_slabs)
+        # what one (page, plane, KV head) holds contiguously, capped at 4 KB: 2 KB on FP8 pages at head_dim 128
+        slab_bytes = min(SLAB_BYTES, TOKENS_PER_PAGE * spec["d"] * self.kv_element_bytes)
+        pool_slabs = self.kv_pools[0].numel() * self.kv_pools[0].element_size() // slab_bytes
+        num_slabs = min(kv_bytes // slab_bytes, pool_slabs)
         order = np.random.Generator(np.random.PCG64(1234)).permutation(pool_slabs)[:num_slabs].astype(np.uint32)
         slab_ids = torch.from_numpy(order.view(np.int32)).to(self.kv_pools[0].device)
         sink = torch.zeros(1, dtype=torch.int32, device=slab_ids.device)
         best = None
         for blocks_per_cu in (2, 4):
             for i in range(3):
-                slab_read(self.kv_pools[i % len(self.kv_pools)], slab_ids, num_slabs, sink, blocks_per_cu)
+                slab_read(self.kv_pools[i % len(self.kv_pools)], slab_ids, num_slabs, sink, blocks_per_cu, 1, slab_bytes)
             pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
             for i, (a, b) in enumerate(pairs):
                 a.record()
-                slab_read(self.kv_pools[i % len(self.kv_pools)], slab_ids, num_slabs, sink, blocks_per_cu)
+                slab_read(self.kv_pools[i % len(self.kv_pools)], slab_ids, num_slabs, sink, blocks_per_cu, 1, slab_bytes)
                 b.record()
             torch.cuda.synchronize()
             mean_us = float(np.mean([a.elapsed_time(b) for a, b in pairs])) * 1e3
             if best is None or mean_us < best["us"]:
                 best = {"us": mean_us, "blocks_per_cu": blocks_per_cu}
-        nbytes = num_slabs * SLAB_BYTES
-        best.update(bytes=int(nbytes), gbps=nbytes / (best["us"] * 1e-6) / 1e9,
-                    what="read-only launch of the workload's K/V bytes as random 4 KB slabs of the same pools, evenly split over a resident grid")
+        nbytes = num_slabs * slab_bytes
+        best.update(bytes=int(nbytes), gbps=nbytes / (best["us"] * 1e-6) / 1e9, slab_bytes=int(slab_bytes),
+                    what=f"read-only launch of the workload's K/V bytes as random {slab_bytes // 1024} KB slabs of the same pools, evenly split over a resident grid")
         return best
 
     def report(self, steps: int, warmup: int) -> dict:

@@ -17,12 +17,15 @@ def test_gpu_reads_listed_slabs_and_leaves_the_sink_alone(device):
     for count in (1, 3, slabs):   # fewer slabs than waves, and a full list
         print(f"bench slab read: {count} slabs", flush=True)
         bench.slab_read(pool, ids, count, sink, blocks_per_cu=2)
+        bench.slab_read(pool, ids, count, sink, blocks_per_cu=2, slab_bytes=2048)   # the first half of the pool, as 2 KB slabs
     torch.cuda.synchronize()
     assert int(sink.item()) == 0
     with pytest.raises(RuntimeError):
         bench.slab_read(pool, ids, 0, sink)          # nothing to read
     with pytest.raises(RuntimeError):
         bench.slab_read(pool, ids, 4, sink, blocks_per_cu=9)
+    with pytest.raises(RuntimeError):
+        bench.slab_read(pool, ids, 4, sink, slab_bytes=1024)
 
 
 def test_bench_aid_library_exports_its_entry_points():

@@ -7,7 +7,8 @@ import bench
 PROFILES = {2: ("split_kv_map_kernel_config2_decode.txt", "split_kv_map_kernel"),
             3: ("split_kv_map_kernel_config3_long_context_gated.txt", "split_kv_map_kernel"),
             4: ("tile_map_kernel_config4_spec_verify.txt", "tile_map_kernel"),
-            5: ("tile_map_kernel_config5_chunked_prefill.txt", "tile_map_kernel")}
+            5: ("tile_map_kernel_config5_chunked_prefill.txt", "tile_map_kernel"),
+            6: ("tile_map_kernel_extra_prefill_d256.txt", "tile_map_kernel")}
 
 
 def test_measured_traffic_constants_match_the_committed_profiles():
