@@ -361,8 +361,8 @@ uint16_t khm_f32_to_bf16(float value);
 float khm_bf16_to_f32(uint16_t bf16_bits);
 /* The same codec on the device, element-wise over `count` values: decode is what the Map kernels apply to FP8 pages
  * (fp8_e4m3x8_to_bf16x8, components/metal/gqa_fp8.metal:1-25), encode is what the page writer applies
- * (bf16_to_fp8_e4m3, components/metal/gqa_kv_page_write.metal:5-31).  `codes` must be 8-byte and `bf16_out` 16-byte
- * aligned for the decoder. */
+ * (bf16_to_fp8_e4m3, components/metal/gqa_kv_page_write.metal:5-31).  The 8-bit buffer (`codes`) must be 8-byte and the
+ * 16-bit buffer (`bf16_out`, `bf16_in`) 16-byte aligned. */
 int khm_fp8_e4m3_to_bf16_device(khm_buffer codes, khm_buffer bf16_out, uint64_t count, void* stream);
 int khm_bf16_to_fp8_e4m3_device(khm_buffer bf16_in, khm_buffer codes, uint64_t count, void* stream);
 

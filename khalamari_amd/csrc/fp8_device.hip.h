@@ -49,18 +49,58 @@ __device__ __forceinline__ uint32_t bf16_bits_to_fp8_e4m3fn(uint32_t bits) {
     return sign | (encoded_exponent << 3) | kept;
 }
 
-// Two bf16 bit patterns (low and high half of `pair`) to their two E4M3FN codes (bits 0..7 and 8..15) through the
-// hardware converter v_cvt_pk_fp8_f32 (round to nearest even, subnormals below 2^-6).  The converter does not
-// saturate by itself, so finite and infinite magnitudes are clamped to 448 first; NaN keeps its sign and becomes 0x7f.
-// Checked against the integer encoder above and the host codec over all 65 536 patterns in both positions.
+// Two bf16 bit patterns (low and high half of `pair`) to their two E4M3FN codes, written to the low (HIGH_HALF = false)
+// or high 16 bits of `old` through v_cvt_scalef32_pk_fp8_bf16 with scale 1 (round to nearest even, subnormals below
+// 2^-6).  The converter does not saturate (magnitudes above 464 come out as the NaN code), so magnitudes are clamped to
+// 448 first, as 16-bit integers on the bf16 fields, which orders finite and infinite magnitudes alike; NaN would be
+// clamped with them and is patched afterwards: it keeps its sign and becomes 0x7f.  Checked against the integer encoder
+// above and the host codec over all 65 536 patterns in every position.
+typedef unsigned short Fp8U16x2 __attribute__((ext_vector_type(2)));
+typedef short Fp8I16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 Fp8Bf16x2 __attribute__((ext_vector_type(2)));
+
+template <bool HIGH_HALF>
+__device__ __forceinline__ uint32_t bf16x2_bits_to_fp8x2_no_nan(uint32_t old, uint32_t pair) {
+    const Fp8U16x2 magnitude = __builtin_bit_cast(Fp8U16x2, pair & 0x7fff7fffu);
+    const Fp8U16x2 limit = {0x43e0, 0x43e0};
+    const uint32_t clamped = (pair & 0x80008000u) | __builtin_bit_cast(uint32_t, __builtin_elementwise_min(magnitude, limit));
+    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(__builtin_bit_cast(Fp8I16x2, old),
+                                                                                 __builtin_bit_cast(Fp8Bf16x2, clamped), 1.0f, HIGH_HALF));
+}
+
+// Nonzero in the half of the result whose half of `pair` is a NaN.
+__device__ __forceinline__ uint32_t bf16x2_nan_halves(uint32_t pair) {
+    const Fp8U16x2 magnitude = __builtin_bit_cast(Fp8U16x2, pair & 0x7fff7fffu);
+    const Fp8U16x2 infinity = {0x7f80, 0x7f80};
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_sub_sat(magnitude, infinity));
+}
+
 __device__ __forceinline__ uint32_t bf16x2_bits_to_fp8x2_e4m3fn(uint32_t pair) {
-    const float low = __uint_as_float(pair << 16), high = __uint_as_float(pair & 0xffff0000u);
-    const float low_clamped = __builtin_amdgcn_fmed3f(low, -448.0f, 448.0f);
-    const float high_clamped = __builtin_amdgcn_fmed3f(high, -448.0f, 448.0f);
-    uint32_t codes = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(low_clamped, high_clamped, 0, false) & 0xffffu;
-    if ((pair & 0x7fffu) > 0x7f80u) codes = (codes & 0xff00u) | ((pair >> 8) & 0x80u) | 0x7fu;
-    if ((pair & 0x7fff0000u) > 0x7f800000u) codes = (codes & 0x00ffu) | ((pair >> 16) & 0x8000u) | 0x7f00u;
+    uint32_t codes = bf16x2_bits_to_fp8x2_no_nan<false>(0u, pair) & 0xffffu;
+    const uint32_t nan = bf16x2_nan_halves(pair);
+    if (nan != 0u) {
+        if ((nan & 0xffffu) != 0u) codes = (codes & 0xff00u) | ((pair >> 8) & 0x80u) | 0x7fu;
+        if ((nan >> 16) != 0u) codes = (codes & 0x00ffu) | ((pair >> 16) & 0x8000u) | 0x7f00u;
+    }
     return codes;
+}
+
+// Four bf16 bit patterns (`first` holds elements 0 and 1, `second` elements 2 and 3) to four codes in element order.
+__device__ __forceinline__ uint32_t bf16x4_bits_to_fp8x4_e4m3fn(uint32_t first, uint32_t second) {
+    uint32_t codes = bf16x2_bits_to_fp8x2_no_nan<true>(bf16x2_bits_to_fp8x2_no_nan<false>(0u, first), second);
+    const uint32_t nan_first = bf16x2_nan_halves(first), nan_second = bf16x2_nan_halves(second);
+    if ((nan_first | nan_second) != 0u) {
+        if ((nan_first & 0xffffu) != 0u) codes = (codes & 0xffffff00u) | ((first >> 8) & 0x80u) | 0x7fu;
+        if ((nan_first >> 16) != 0u) codes = (codes & 0xffff00ffu) | ((first >> 16) & 0x8000u) | 0x7f00u;
+        if ((nan_second & 0xffffu) != 0u) codes = (codes & 0xff00ffffu) | ((second << 8) & 0x800000u) | 0x7f0000u;
+        if ((nan_second >> 16) != 0u) codes = (codes & 0x00ffffffu) | (second & 0x80000000u) | 0x7f000000u;
+    }
+    return codes;
+}
+
+// Eight bf16 bit patterns to eight codes, element order preserved.
+__device__ __forceinline__ uint2 bf16x8_bits_to_fp8x8_e4m3fn(uint4 bits) {
+    return make_uint2(bf16x4_bits_to_fp8x4_e4m3fn(bits.x, bits.y), bf16x4_bits_to_fp8x4_e4m3fn(bits.z, bits.w));
 }
 
 }  // namespace khm

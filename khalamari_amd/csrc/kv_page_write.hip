@@ -44,10 +44,7 @@ __global__ __launch_bounds__(1024) void kv_page_write_kernel(const PageWritePara
         const uint4 k = *reinterpret_cast<const uint4*>(p.flat_k + source);
         const uint4 v = *reinterpret_cast<const uint4*>(p.flat_v + source);
         if constexpr (FP8_PAGES) {
-            auto encode8 = [](uint4 bits) {
-                return make_uint2(bf16x2_bits_to_fp8x2_e4m3fn(bits.x) | (bf16x2_bits_to_fp8x2_e4m3fn(bits.y) << 16),
-                                  bf16x2_bits_to_fp8x2_e4m3fn(bits.z) | (bf16x2_bits_to_fp8x2_e4m3fn(bits.w) << 16));
-            };
+            auto encode8 = [](uint4 bits) { return bf16x8_bits_to_fp8x8_e4m3fn(bits); };
             *reinterpret_cast<uint2*>(k_target) = encode8(k);
             *reinterpret_cast<uint2*>(v_target) = encode8(v);
         } else {
@@ -80,18 +77,22 @@ __global__ __launch_bounds__(256) void fp8_decode_kernel(const uint8_t* codes, u
     for (uint64_t i = gid; i < count; ++i) bf16_out[i] = (uint16_t)(fp8x2_to_bf16x2<false>(codes[i]) & 0xffffu);
 }
 
-// Thread t encodes elements 2t and 2t+1 with the paired hardware conversion the page writer uses; a last odd element
-// takes the integer encoder.
+// Thread t encodes elements 8t .. 8t+7 with the eight-wide conversion the page writers use; what is left of the last
+// group goes through the paired conversion, and a last odd element through the integer encoder.
 __global__ __launch_bounds__(256) void fp8_encode_kernel(const uint16_t* bf16_in, uint8_t* codes, uint64_t count) {
-    const uint64_t gid = ((uint64_t)blockIdx.x * 256 + threadIdx.x) * 2;
-    if (gid + 1 < count) {
-        const uint32_t pair = (uint32_t)bf16_in[gid] | ((uint32_t)bf16_in[gid + 1] << 16);
-        const uint32_t both = bf16x2_bits_to_fp8x2_e4m3fn(pair);
-        codes[gid] = (uint8_t)(both & 0xffu);
-        codes[gid + 1] = (uint8_t)(both >> 8);
-    } else if (gid < count) {
-        codes[gid] = (uint8_t)bf16_bits_to_fp8_e4m3fn(bf16_in[gid]);
+    const uint64_t gid = ((uint64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (gid >= count) return;
+    if (gid + 8 <= count) {
+        *reinterpret_cast<uint2*>(codes + gid) = bf16x8_bits_to_fp8x8_e4m3fn(*reinterpret_cast<const uint4*>(bf16_in + gid));
+        return;
     }
+    uint64_t i = gid;
+    for (; i + 1 < count; i += 2) {
+        const uint32_t both = bf16x2_bits_to_fp8x2_e4m3fn((uint32_t)bf16_in[i] | ((uint32_t)bf16_in[i + 1] << 16));
+        codes[i] = (uint8_t)(both & 0xffu);
+        codes[i + 1] = (uint8_t)(both >> 8);
+    }
+    if (i < count) codes[i] = (uint8_t)bf16_bits_to_fp8_e4m3fn(bf16_in[i]);
 }
 
 static DeviceReplayU32 to_device_replay(khm_replay_u32 value) { return DeviceReplayU32{value.is_parameter, value.value}; }
@@ -226,7 +227,10 @@ extern "C" int khm_bf16_to_fp8_e4m3_device(khm_buffer bf16_in, khm_buffer codes,
                 (unsigned long long)bf16_in.len_bytes, (unsigned long long)(count * 2));
     KHM_REQUIRE(codes.ptr != nullptr && codes.len_bytes >= count, "codes buffer holds %llu bytes, needs %llu",
                 (unsigned long long)codes.len_bytes, (unsigned long long)count);
-    hipLaunchKernelGGL(fp8_encode_kernel, dim3((uint32_t)(((count + 1) / 2 + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+    KHM_REQUIRE(reinterpret_cast<uintptr_t>(codes.ptr) % 8 == 0 && reinterpret_cast<uintptr_t>(bf16_in.ptr) % 16 == 0,
+                "FP8 encode buffers must be 8- and 16-byte aligned");
+    const uint64_t threads = (count + 7) / 8;
+    hipLaunchKernelGGL(fp8_encode_kernel, dim3((uint32_t)((threads + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint16_t*>(bf16_in.ptr), static_cast<uint8_t*>(codes.ptr), count);
     return check_page_write_launch("FP8 encode");
 }

@@ -204,12 +204,23 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
         for (int i = 0; i < 8; ++i) x[j][i] = 0.0f;
         if (valid[j]) Row8<T>::load(static_cast<const T*>(p.input) + ((uint64_t)tokens[j] * p.num_heads + heads[j]) * p.head_dim + first, x[j]);
     }
+    // Page writes: the V chunks and the page-table walk (request slot, position -> page id) of every row are requested
+    // here, beside the K rows, so that their round trips pass under the sine/cosine evaluation and the block barrier
+    // instead of standing between the last arithmetic and the stores.
     uint4 v_chunk[PAGES != 0 ? kRowsInFlight : 1];
+    PageTarget target[PAGES != 0 ? kRowsInFlight : 1];
     if constexpr (PAGES != 0) {
+        constexpr uint32_t kElementBytes = PAGES == 2 ? 1 : 2;
+        const uint32_t layer = resolve_u32(pages->layer_index, pages->replay_parameters);
 #pragma unroll
         for (int j = 0; j < kRowsInFlight; ++j) {
             v_chunk[j] = make_uint4(0, 0, 0, 0);
-            if (valid[j]) v_chunk[j] = *reinterpret_cast<const uint4*>(pages->flat_v + ((uint64_t)tokens[j] * p.num_heads + heads[j]) * p.head_dim + first);
+            target[j] = PageTarget{0, 0};
+            if (valid[j]) {
+                v_chunk[j] = *reinterpret_cast<const uint4*>(pages->flat_v + ((uint64_t)tokens[j] * p.num_heads + heads[j]) * p.head_dim + first);
+                target[j] = page_target_of(*pages, pages->req_slots[tokens[j]], pages->flat_token_indices[tokens[j]], layer, heads[j], first,
+                                           kElementBytes);
+            }
         }
     }
     // the rotation tables of the block's tokens, one sine/cosine evaluation per token and rotary pair
@@ -271,20 +282,14 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
             Row8<T>::store(static_cast<T*>(p.output) + ((uint64_t)tokens[j] * p.num_heads + heads[j]) * p.head_dim + first, out);
         } else {
             const uint4 k_chunk = make_uint4(pack_bf16x2(out[0], out[1]), pack_bf16x2(out[2], out[3]), pack_bf16x2(out[4], out[5]), pack_bf16x2(out[6], out[7]));
-            constexpr uint32_t kElementBytes = PAGES == 2 ? 1 : 2;
-            const PageTarget target = page_target_of(*pages, pages->req_slots[tokens[j]], pages->flat_token_indices[tokens[j]],
-                                                     resolve_u32(pages->layer_index, pages->replay_parameters), heads[j], first, kElementBytes);
-            uint8_t* k_target = pages->pages + target.k_offset;
+            uint8_t* k_target = pages->pages + target[j].k_offset;
             if constexpr (PAGES == 2) {
-                auto encode8 = [](uint4 bits) {
-                    return make_uint2(bf16x2_bits_to_fp8x2_e4m3fn(bits.x) | (bf16x2_bits_to_fp8x2_e4m3fn(bits.y) << 16),
-                                      bf16x2_bits_to_fp8x2_e4m3fn(bits.z) | (bf16x2_bits_to_fp8x2_e4m3fn(bits.w) << 16));
-                };
+                auto encode8 = [](uint4 bits) { return bf16x8_bits_to_fp8x8_e4m3fn(bits); };
                 *reinterpret_cast<uint2*>(k_target) = encode8(k_chunk);
-                *reinterpret_cast<uint2*>(k_target + target.v_distance) = encode8(v_chunk[j]);
+                *reinterpret_cast<uint2*>(k_target + target[j].v_distance) = encode8(v_chunk[j]);
             } else {
                 *reinterpret_cast<uint4*>(k_target) = k_chunk;
-                *reinterpret_cast<uint4*>(k_target + target.v_distance) = v_chunk[j];
+                *reinterpret_cast<uint4*>(k_target + target[j].v_distance) = v_chunk[j];
             }
         }
     }

@@ -93,12 +93,16 @@ def test_gpu_fp8_codec_matches_the_host_codec_exhaustively():
     encoded = torch.zeros(65536, dtype=torch.uint8, device=device)
     kpw.fp8_encode_device(every_bf16, encoded, 65536)
     assert np.array_equal(encoded.cpu().numpy(), oracle.bf16_bits_to_fp8(np.arange(65536, dtype=np.uint32).astype(np.uint16)))
-    # the device encoder converts elements in pairs: every pattern also in the other half of a pair, and an odd count
-    rolled = np.roll(np.arange(65536, dtype=np.uint32).astype(np.uint16), 1)[:65535]
-    encoded = torch.full((65536,), 0xAA, dtype=torch.uint8, device=device)
-    kpw.fp8_encode_device(torch.from_numpy(rolled.view(np.int16).copy()).to(device), encoded, 65535)
-    got = encoded.cpu().numpy()
-    assert np.array_equal(got[:65535], oracle.bf16_bits_to_fp8(rolled)) and got[65535] == 0xAA
+    # the device encoder converts eight elements at a time (pairs and a single element at the end of an odd count): every
+    # pattern in every position of a group, and counts that leave 7 .. 1 elements to the tail paths
+    every = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    for shift in range(1, 9):
+        rolled = np.roll(every, shift)[:65536 - shift]
+        encoded = torch.full((65536,), 0xAA, dtype=torch.uint8, device=device)
+        kpw.fp8_encode_device(torch.from_numpy(rolled.view(np.int16).copy()).to(device), encoded, rolled.size)
+        got = encoded.cpu().numpy()
+        assert np.array_equal(got[:rolled.size], oracle.bf16_bits_to_fp8(rolled)), shift
+        assert np.all(got[rolled.size:] == 0xAA), shift
 
 
 def _run_page_write(device, config, shape, pages, flat_k, flat_v, req_slots, tokens, page_ids, active, layer=0, parameters=None):
