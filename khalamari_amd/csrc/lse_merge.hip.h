@@ -34,12 +34,11 @@ __device__ __forceinline__ uint64_t merge_load_u64(const void* address) {
 
 // Merges partials first, first + step, ... < end of one (Q head, token offset) row into `state`, for the four
 // dims chunk*4 .. chunk*4+3.  `safe_part` is any valid partial index (address of masked-off batch slots).
-template <int D, bool COHERENT>
+template <int D, bool COHERENT, int BATCH = 8>
 __device__ __forceinline__ void merge_partial_slice(MergeState& state, const float* max_logits, const float* exp_sums, const void* partial,
                                                     bool f32_partials, uint32_t first, uint32_t end, uint32_t step, uint32_t safe_part,
                                                     uint32_t num_q_heads, uint32_t q_head, uint32_t max_q_tokens, uint32_t token_offset,
                                                     int chunk) {
-    constexpr int BATCH = 8;
     for (; first < end; first += BATCH * step) {
         float part_max[BATCH], part_sum[BATCH];
         uint64_t lo[BATCH], hi[BATCH];

@@ -73,8 +73,8 @@ __global__ __launch_bounds__(kReduceThreads) void split_kv_reduce_kernel(const R
 }
 
 // The same merge for rows with few partials (speculative-verify tiles have about ten): a group of D/4 threads owns one
-// (token, head) row and walks all of its partials itself, eight loads in flight, so a block serves 256 / (D/4) rows
-// and nothing passes through LDS.  Rows are numbered (unit * max_q_tokens + token slot) * num_q_heads + head.
+// (token, head) row and walks all of its partials itself, sixteen loads in flight (a row of a decode batch with 512-token
+// partitions has up to sixteen partials), so a block serves 256 / (D/4) rows and nothing passes through LDS.  Rows are numbered (unit * max_q_tokens + token slot) * num_q_heads + head.
 template <int D, bool RANGED>
 __global__ __launch_bounds__(kReduceThreads) void split_kv_reduce_rows_kernel(const ReduceParams p) {
     constexpr int CHUNKS = D / 4;
@@ -98,7 +98,7 @@ __global__ __launch_bounds__(kReduceThreads) void split_kv_reduce_rows_kernel(co
     const uint32_t end = p.cu_partial_outputs[unit + 1];
     MergeState state = merge_state_empty();
     if (end > begin) {
-        merge_partial_slice<D, false>(state, p.max_logits, p.exp_sums, p.partial, p.partial_is_f32 != 0, begin, end, 1, begin, p.num_q_heads, head,
+        merge_partial_slice<D, false, 16>(state, p.max_logits, p.exp_sums, p.partial, p.partial_is_f32 != 0, begin, end, 1, begin, p.num_q_heads, head,
                                       max_q, local, chunk);
     }
     const uint64_t out_index = ((uint64_t)(flat_begin + local) * p.num_q_heads + head) * D + chunk * 4;

@@ -105,6 +105,14 @@ template <typename T>
 struct Row8;
 template <>
 struct Row8<float> {
+    struct Raw { float4 a, b; };
+    static __device__ __forceinline__ Raw zero() { return Raw{make_float4(0.f, 0.f, 0.f, 0.f), make_float4(0.f, 0.f, 0.f, 0.f)}; }
+    static __device__ __forceinline__ Raw load_raw(const float* source) {
+        return Raw{*reinterpret_cast<const float4*>(source), *reinterpret_cast<const float4*>(source + 4)};
+    }
+    static __device__ __forceinline__ void unpack(const Raw& raw, float (&x)[8]) {
+        x[0] = raw.a.x, x[1] = raw.a.y, x[2] = raw.a.z, x[3] = raw.a.w, x[4] = raw.b.x, x[5] = raw.b.y, x[6] = raw.b.z, x[7] = raw.b.w;
+    }
     static __device__ __forceinline__ void load(const float* source, float (&x)[8]) {
         const float4 a = *reinterpret_cast<const float4*>(source), b = *reinterpret_cast<const float4*>(source + 4);
         x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w, x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
@@ -116,6 +124,14 @@ struct Row8<float> {
 };
 template <>
 struct Row8<uint16_t> {
+    typedef uint4 Raw;
+    static __device__ __forceinline__ Raw zero() { return make_uint4(0u, 0u, 0u, 0u); }
+    static __device__ __forceinline__ Raw load_raw(const uint16_t* source) { return *reinterpret_cast<const uint4*>(source); }
+    static __device__ __forceinline__ void unpack(const Raw& v, float (&x)[8]) {
+        const uint32_t words[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[2 * i] = __uint_as_float(words[i] << 16), x[2 * i + 1] = __uint_as_float(words[i] & 0xffff0000u);
+    }
     static __device__ __forceinline__ void load(const uint16_t* source, float (&x)[8]) {
         const uint4 v = *reinterpret_cast<const uint4*>(source);
         const uint32_t words[4] = {v.x, v.y, v.z, v.w};
@@ -190,7 +206,7 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
     const bool lower = first < rope_half, rotated = first < p.rope_dim;
     const int partner_lane = ((int)lane + (lower ? (int)(rope_half / 8) : -(int)(rope_half / 8))) & 63;
 
-    float x[kRowsInFlight][8];
+    typename Row8<T>::Raw raw[kRowsInFlight];   // rows stay as loaded until their turn: half the registers of eight floats
     uint32_t heads[kRowsInFlight], tokens[kRowsInFlight], local_tokens[kRowsInFlight];
     bool valid[kRowsInFlight];
 #pragma unroll
@@ -200,9 +216,8 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
         tokens[j] = first_token + local_tokens[j];
         heads[j] = blockIdx.y * kRowSlots + (slot & ((1u << slot_shift) - 1u));
         valid[j] = holds && heads[j] < p.num_heads && local_tokens[j] < tokens_per_block && tokens[j] < num_active_tokens;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) x[j][i] = 0.0f;
-        if (valid[j]) Row8<T>::load(static_cast<const T*>(p.input) + ((uint64_t)tokens[j] * p.num_heads + heads[j]) * p.head_dim + first, x[j]);
+        raw[j] = Row8<T>::zero();
+        if (valid[j]) raw[j] = Row8<T>::load_raw(static_cast<const T*>(p.input) + ((uint64_t)tokens[j] * p.num_heads + heads[j]) * p.head_dim + first);
     }
     // Page writes: the V chunks and the page-table walk (request slot, position -> page id) of every row are requested
     // here, beside the K rows, so that their round trips pass under the sine/cosine evaluation and the block barrier
@@ -233,10 +248,8 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
             sincosf(position * p.inverse_frequencies[pair], &sines[local * rope_half + pair], &cosines[local * rope_half + pair]);
         }
     }
-    float w[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) w[i] = 0.0f;
-    if (holds) Row8<W>::load(static_cast<const W*>(p.norm_weight) + first, w);
+    typename Row8<W>::Raw w_raw = Row8<W>::zero();
+    if (holds) w_raw = Row8<W>::load_raw(static_cast<const W*>(p.norm_weight) + first);
     __syncthreads();
     const float inverse_dim = 1.0f / (float)p.head_dim;
     float sine[8], cosine[8];
@@ -244,9 +257,12 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
     for (int i = 0; i < 8; ++i) sine[i] = 0.0f, cosine[i] = 1.0f;
 #pragma unroll
     for (int j = 0; j < kRowsInFlight; ++j) {
+        float x[8], w[8];
+        Row8<T>::unpack(raw[j], x);
+        Row8<W>::unpack(w_raw, w);
         float acc = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc += x[j][i] * x[j][i];
+        for (int i = 0; i < 8; ++i) acc += x[i] * x[i];
         acc = sum_in_row<LPR>(acc, lane);
         // v_rsq_f32 (1 ulp) and one Newton step, which leaves the error below that of a correctly rounded rsqrt's input
         const float mean = acc * inverse_dim + p.eps;
@@ -262,9 +278,9 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
         for (int i = 0; i < 8; ++i) {
             float normed;
             if constexpr (sizeof(T) == 2 && sizeof(W) == 2) {
-                normed = round_to_bf16(w[i] * round_to_bf16(x[j][i] * inv_rms));
+                normed = round_to_bf16(w[i] * round_to_bf16(x[i] * inv_rms));
             } else {
-                normed = w[i] * x[j][i] * inv_rms;
+                normed = w[i] * x[i] * inv_rms;
             }
             float partner;
             if constexpr (PARTNER == 8) partner = dpp_move<0x128>(normed);          // row_ror:8 = lane ^ 8 inside a 16-lane row
