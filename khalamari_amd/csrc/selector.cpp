@@ -310,10 +310,7 @@ static int lookup_variant(const khm_sdpa_config& config, uint32_t queries, khm_s
     // LDS feeds as many MFMA columns as possible.  Narrower blocks are bandwidth-bound and stay on small tiles.
     // At D 256 the 256-column tile does not fit the register file (it spills): tiles stop at 192 columns (twelve waves of
     // one column tile: 32 tokens x 6 heads of a group-6 model) and otherwise at 128.
-#ifndef KHM_D256_PREFILL_COLUMNS
-#define KHM_D256_PREFILL_COLUMNS (3 * kMaxPrefillColumns / 4)
-#endif
-    const uint32_t prefill_columns = config.head_dim > 128 ? KHM_D256_PREFILL_COLUMNS : kMaxPrefillColumns;
+    const uint32_t prefill_columns = config.head_dim > 128 ? 3 * kMaxPrefillColumns / 4 : kMaxPrefillColumns;
     const uint32_t max_columns = queries >= 16 ? prefill_columns : kMaxColumns;
     uint32_t heads = std::min(ratio, max_columns);
     uint32_t tile = queries;
