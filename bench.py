@@ -31,7 +31,7 @@ NUM_POOLS = 3
 # HBM bytes per Map launch from the hardware counters, (FETCH_SIZE * 2.000 + WRITE_SIZE * 1.000) KiB per dispatch:
 # two `rocprofv3 --pmc` runs per config, each counter scaled by what it reads for a plain 1 GiB copy kernel
 # (`--calibration-copy`).  The summaries with their commands are the text files under profiles/.
-MEASURED_MAP_TRAFFIC_BYTES = {2: 564_443_136, 3: 2_151_780_352, 4: 1_447_216_128, 5: 1_202_862_080, 6: 1_068_921_856}
+MEASURED_MAP_TRAFFIC_BYTES = {2: 564_434_944, 3: 2_151_780_352, 4: 1_447_223_296, 5: 1_202_804_736, 6: 1_068_930_048}
 
 CONFIGS = {
     1: dict(name="config1: B=1 q=1 Hq32/Hkv8/D128 ctx 1024, identity pages", hq=32, hkv=8, d=128, kind="decode", kv_slice=64),
