@@ -32,6 +32,7 @@ NUM_POOLS = 3
 # two `rocprofv3 --pmc` runs per config, each counter scaled by what it reads for a plain 1 GiB copy kernel
 # (`--calibration-copy`).  The summaries with their commands are the text files under profiles/.
 MEASURED_MAP_TRAFFIC_BYTES = {2: 564_434_944, 3: 2_151_780_352, 4: 1_447_223_296, 5: 1_202_804_736, 6: 1_068_930_048}
+MEASURED_MAP_TRAFFIC_BYTES_FP8_PAGES = {2: 285_208_576, 3: 1_077_938_176, 4: 729_363_456, 5: 869_689_344, 6: 1_614_070_784}
 
 CONFIGS = {
     1: dict(name="config1: B=1 q=1 Hq32/Hkv8/D128 ctx 1024, identity pages", hq=32, hkv=8, d=128, kind="decode", kv_slice=64),
@@ -686,7 +687,7 @@ def main() -> int:
             "peak": MFMA_BF16_PEAK_TFLOPS if prefill else HBM_PEAK_GBPS,
             "unit": "TFLOP/s" if prefill else "GB/s",
             "frac": head["roofline_frac"],
-            "traffic": None if args.fp8_pages else MEASURED_MAP_TRAFFIC_BYTES.get(args.config),
+            "traffic": (MEASURED_MAP_TRAFFIC_BYTES_FP8_PAGES if args.fp8_pages else MEASURED_MAP_TRAFFIC_BYTES).get(args.config),
             "kernel": head["map_kernel"],
             "kernel_us": head["map_kernel_us"],
             "algorithmic_bytes": head.get("algorithmic_bytes"),

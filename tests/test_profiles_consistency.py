@@ -12,7 +12,10 @@ PROFILES = {2: ("split_kv_map_kernel_config2_decode.txt", "split_kv_map_kernel")
 
 
 def test_measured_traffic_constants_match_the_committed_profiles():
-    for index, (name, kernel) in PROFILES.items():
+    cases = [(index, name, kernel, bench.MEASURED_MAP_TRAFFIC_BYTES) for index, (name, kernel) in PROFILES.items()]
+    cases += [(index, name.replace(".txt", "_fp8_pages.txt"), kernel, bench.MEASURED_MAP_TRAFFIC_BYTES_FP8_PAGES)
+              for index, (name, kernel) in PROFILES.items()]
+    for index, name, kernel, constants in cases:
         text = open(os.path.join(bench.ROOT, "profiles", name)).read()
         factors = re.search(r"scale factors ([\d.]+) \(FETCH_SIZE\) and ([\d.]+) \(WRITE_SIZE\)", text)
         assert factors, name
@@ -21,4 +24,4 @@ def test_measured_traffic_constants_match_the_committed_profiles():
         assert row, name
         measured = (int(row.group(1)) * fetch_factor + int(row.group(2)) * write_factor) * 1024
         # the scale factors are printed with three decimals
-        assert abs(measured - bench.MEASURED_MAP_TRAFFIC_BYTES[index]) <= 1e-3 * measured, (index, measured)
+        assert abs(measured - constants[index]) <= 1e-3 * measured, (name, measured)
