@@ -180,6 +180,7 @@ __device__ __forceinline__ float sum_in_row(float v, uint32_t lane) {
 // of ONE token: the first lanes evaluate the token's sines and cosines once into LDS, and each wave issues the loads
 // of up to kRowsInFlight row groups before it uses the first.
 constexpr int kRowsInFlight = 4;
+constexpr int kPageRowsInFlight = 2;   // the fused page writer: 64 instead of 90 registers, eight waves per SIMD, twice the blocks
 constexpr int kMaxTokensPerBlock = 16;
 
 // PAGES: 0 writes the rows to p.output; 1 / 2 scatter them, as K rows, straight into bf16 / FP8 E4M3FN pages through
@@ -189,7 +190,8 @@ template <typename T, typename W, uint32_t LPR, uint32_t PARTNER, int PAGES>
 __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, const PageWriteParams* pages) {
     static_assert(PAGES == 0 || sizeof(T) == 2, "pages are written from bf16 rows");
     constexpr uint32_t kRowsPerWave = 64u / LPR;
-    constexpr uint32_t kRowSlots = 4 * kRowsInFlight * kRowsPerWave;   // (token, head) rows a block holds
+    constexpr int kRows = PAGES != 0 ? kPageRowsInFlight : kRowsInFlight;   // row groups of a wave
+    constexpr uint32_t kRowSlots = 4 * kRows * kRowsPerWave;   // (token, head) rows a block holds
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
     // Row slot s of the block belongs to token s >> shift of the block's tokens and to head s & (2^shift - 1) of this
@@ -206,11 +208,11 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
     const bool lower = first < rope_half, rotated = first < p.rope_dim;
     const int partner_lane = ((int)lane + (lower ? (int)(rope_half / 8) : -(int)(rope_half / 8))) & 63;
 
-    typename Row8<T>::Raw raw[kRowsInFlight];   // rows stay as loaded until their turn: half the registers of eight floats
-    uint32_t heads[kRowsInFlight], tokens[kRowsInFlight], local_tokens[kRowsInFlight];
-    bool valid[kRowsInFlight];
+    typename Row8<T>::Raw raw[kRows];   // rows stay as loaded until their turn: half the registers of eight floats
+    uint32_t heads[kRows], tokens[kRows], local_tokens[kRows];
+    bool valid[kRows];
 #pragma unroll
-    for (int j = 0; j < kRowsInFlight; ++j) {
+    for (int j = 0; j < kRows; ++j) {
         const uint32_t slot = (j * 4 + wave) * kRowsPerWave + sub_row;
         local_tokens[j] = slot >> slot_shift;
         tokens[j] = first_token + local_tokens[j];
@@ -222,13 +224,13 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
     // Page writes: the V chunks and the page-table walk (request slot, position -> page id) of every row are requested
     // here, beside the K rows, so that their round trips pass under the sine/cosine evaluation and the block barrier
     // instead of standing between the last arithmetic and the stores.
-    uint4 v_chunk[PAGES != 0 ? kRowsInFlight : 1];
-    PageTarget target[PAGES != 0 ? kRowsInFlight : 1];
+    uint4 v_chunk[PAGES != 0 ? kRows : 1];
+    PageTarget target[PAGES != 0 ? kRows : 1];
     if constexpr (PAGES != 0) {
         constexpr uint32_t kElementBytes = PAGES == 2 ? 1 : 2;
         const uint32_t layer = resolve_u32(pages->layer_index, pages->replay_parameters);
 #pragma unroll
-        for (int j = 0; j < kRowsInFlight; ++j) {
+        for (int j = 0; j < kRows; ++j) {
             v_chunk[j] = make_uint4(0, 0, 0, 0);
             target[j] = PageTarget{0, 0};
             if (valid[j]) {
@@ -256,7 +258,7 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
 #pragma unroll
     for (int i = 0; i < 8; ++i) sine[i] = 0.0f, cosine[i] = 1.0f;
 #pragma unroll
-    for (int j = 0; j < kRowsInFlight; ++j) {
+    for (int j = 0; j < kRows; ++j) {
         float x[8], w[8];
         Row8<T>::unpack(raw[j], x);
         Row8<W>::unpack(w_raw, w);
@@ -467,11 +469,11 @@ struct RowsGeometry {
     uint32_t lanes_per_row, partner, tokens_per_block, slot_shift;
     dim3 grid;
 };
-static RowsGeometry rows_geometry(const khm_rms_norm_rope_config& config, uint32_t num_total_tokens, uintptr_t address_bits) {
+static RowsGeometry rows_geometry(const khm_rms_norm_rope_config& config, uint32_t num_total_tokens, uintptr_t address_bits, int rows_in_flight = kRowsInFlight) {
     RowsGeometry g{};
     g.fits = address_bits % 16 == 0 && config.head_dim <= 512 && config.head_dim % 8 == 0 && (config.rope_dim / 2) % 8 == 0;
     g.lanes_per_row = config.head_dim <= 64 ? 8u : (config.head_dim <= 128 ? 16u : (config.head_dim <= 256 ? 32u : 64u));
-    const uint32_t row_slots = 4 * kRowsInFlight * (64u / g.lanes_per_row);   // a power of two
+    const uint32_t row_slots = 4 * (uint32_t)rows_in_flight * (64u / g.lanes_per_row);   // a power of two
     // few heads: a token takes the next power of two of row slots and a block serves several tokens
     uint32_t slots_per_token = 1;
     while (slots_per_token < config.num_heads && slots_per_token < row_slots) slots_per_token *= 2;
@@ -553,7 +555,7 @@ extern "C" int khm_k_norm_rope_page_write(const khm_rms_norm_rope_config* norm_c
                                                buffers->flat_token_indices, nullptr, num_active_tokens, replay_parameters, &p))
         return status;
     const RowsGeometry geometry = rows_geometry(*norm_config, shape->num_total_token_writes,
-                                                (uintptr_t)p.input | (uintptr_t)pages.flat_v | (uintptr_t)p.norm_weight | (uintptr_t)pages.pages);
+                                                (uintptr_t)p.input | (uintptr_t)pages.flat_v | (uintptr_t)p.norm_weight | (uintptr_t)pages.pages, kPageRowsInFlight);
     if (!geometry.fits || page_config->page_bytes % 16 != 0)
         return fail(KHM_ERR_UNSUPPORTED, "the fused K RMSNorm/RoPE page write needs 16-byte aligned buffers, head_dim <= 512, and head_dim and "
                                          "rope_dim / 2 multiples of 8: run khm_rms_norm_rope and khm_kv_page_write instead");
