@@ -28,7 +28,11 @@ __global__ __launch_bounds__(256) void calibration_slab_read_kernel(const unsign
         const uint64_t first = ((uint64_t)slab_ids[slab >> run_shift] << run_shift) + (slab & ((1u << run_shift) - 1u));
         const unsigned char* base = pool + first * SLAB + row * ROW + group * 16;
 #pragma unroll
-        for (int i = 0; i < LOADS; ++i) target[i] = *reinterpret_cast<const uint4*>(base + i * 64);
+        for (int i = 0; i < LOADS; ++i) {   // streaming (nt) loads, as the Map kernels issue for bytes nobody reads twice
+            typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
+            const U32x4 v = __builtin_nontemporal_load(reinterpret_cast<const U32x4*>(base + i * 64));
+            target[i] = make_uint4(v[0], v[1], v[2], v[3]);
+        }
     };
     auto fold = [&](const uint4 (&source)[LOADS]) {
 #pragma unroll

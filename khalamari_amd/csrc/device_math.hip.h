@@ -88,6 +88,26 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
 
+// Streaming accesses (nt): bytes that are written once for a later launch, or read once by this block and by no other.
+// They take no room in the XCD's L2 from data that is used again.  Measured on the decode Map: 107 -> 98 us on a
+// 32-request batch; on the verify tiles 240 -> 223 us; on RMSNorm + RoPE rows 102 -> 86 us with streaming stores (and
+// 94 us with streaming loads as well, so its loads stay ordinary ones).
+__device__ __forceinline__ void store_streaming(void* target, uint4 value) {
+    typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
+    const U32x4 v = {value.x, value.y, value.z, value.w};
+    __builtin_nontemporal_store(v, reinterpret_cast<U32x4*>(target));
+}
+__device__ __forceinline__ void store_streaming(void* target, uint2 value) {
+    typedef uint32_t U32x2 __attribute__((ext_vector_type(2)));
+    const U32x2 v = {value.x, value.y};
+    __builtin_nontemporal_store(v, reinterpret_cast<U32x2*>(target));
+}
+__device__ __forceinline__ uint4 load_streaming(const void* source) {
+    typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
+    const U32x4 v = __builtin_nontemporal_load(reinterpret_cast<const U32x4*>(source));
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
+
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits) { return __uint_as_float(bits << 16); }
 
 // Round-to-nearest-even f32 -> bf16 bits (v_cvt_pk_bf16_f32 on gfx950).

@@ -45,11 +45,11 @@ __global__ __launch_bounds__(1024) void kv_page_write_kernel(const PageWritePara
         const uint4 v = *reinterpret_cast<const uint4*>(p.flat_v + source);
         if constexpr (FP8_PAGES) {
             auto encode8 = [](uint4 bits) { return bf16x8_bits_to_fp8x8_e4m3fn(bits); };
-            *reinterpret_cast<uint2*>(k_target) = encode8(k);
-            *reinterpret_cast<uint2*>(v_target) = encode8(v);
+            store_streaming(k_target, encode8(k));
+            store_streaming(v_target, encode8(v));
         } else {
-            *reinterpret_cast<uint4*>(k_target) = k;
-            *reinterpret_cast<uint4*>(v_target) = v;
+            store_streaming(k_target, k);
+            store_streaming(v_target, v);
         }
         return;
     }

@@ -118,8 +118,10 @@ struct Row8<float> {
         x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w, x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
     }
     static __device__ __forceinline__ void store(float* target, const float (&x)[8]) {
-        *reinterpret_cast<float4*>(target) = make_float4(x[0], x[1], x[2], x[3]);
-        *reinterpret_cast<float4*>(target + 4) = make_float4(x[4], x[5], x[6], x[7]);
+        typedef float F32x4 __attribute__((ext_vector_type(4)));
+        const F32x4 low = {x[0], x[1], x[2], x[3]}, high = {x[4], x[5], x[6], x[7]};
+        __builtin_nontemporal_store(low, reinterpret_cast<F32x4*>(target));
+        __builtin_nontemporal_store(high, reinterpret_cast<F32x4*>(target + 4));
     }
 };
 template <>
@@ -139,7 +141,9 @@ struct Row8<uint16_t> {
         for (int i = 0; i < 4; ++i) x[2 * i] = __uint_as_float(words[i] << 16), x[2 * i + 1] = __uint_as_float(words[i] & 0xffff0000u);
     }
     static __device__ __forceinline__ void store(uint16_t* target, const float (&x)[8]) {
-        *reinterpret_cast<uint4*>(target) = make_uint4(pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3]), pack_bf16x2(x[4], x[5]), pack_bf16x2(x[6], x[7]));
+        typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
+        const U32x4 packed = {pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3]), pack_bf16x2(x[4], x[5]), pack_bf16x2(x[6], x[7])};
+        __builtin_nontemporal_store(packed, reinterpret_cast<U32x4*>(target));   // written once, read by a later launch
     }
 };
 
@@ -303,11 +307,11 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
             uint8_t* k_target = pages->pages + target[j].k_offset;
             if constexpr (PAGES == 2) {
                 auto encode8 = [](uint4 bits) { return bf16x8_bits_to_fp8x8_e4m3fn(bits); };
-                *reinterpret_cast<uint2*>(k_target) = encode8(k_chunk);
-                *reinterpret_cast<uint2*>(k_target + target[j].v_distance) = encode8(v_chunk[j]);
+                store_streaming(k_target, encode8(k_chunk));
+                store_streaming(k_target + target[j].v_distance, encode8(v_chunk[j]));
             } else {
-                *reinterpret_cast<uint4*>(k_target) = k_chunk;
-                *reinterpret_cast<uint4*>(k_target + target[j].v_distance) = v_chunk[j];
+                store_streaming(k_target, k_chunk);
+                store_streaming(k_target + target[j].v_distance, v_chunk[j]);
             }
         }
     }

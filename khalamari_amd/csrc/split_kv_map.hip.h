@@ -272,7 +272,7 @@ __global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapPara
             const uint64_t page = (row >= 8 ? id1 : id0);
             const unsigned char* base = p.kv_pages + page * p.page_bytes + kv_head_row0_k + (uint64_t)in_page * ROW_BYTES + g * 16;
 #pragma unroll
-            for (int i = 0; i < LOADS; ++i) tile.k[i] = *reinterpret_cast<const uint4*>(base + i * 64);
+            for (int i = 0; i < LOADS; ++i) tile.k[i] = load_streaming(base + i * 64);   // this block is the only reader
         }
         {
             const uint32_t row_in_load = lane / LANES_PER_ROW;
@@ -283,7 +283,7 @@ __global__ __launch_bounds__(NWAVES * 64) void split_kv_map_kernel(const MapPara
                 const uint32_t in_page = (first_token + row) & (tpp - 1);
                 const uint64_t page = (row >= 8 ? id1 : id0);
                 const unsigned char* source = p.kv_pages + page * p.page_bytes + kv_head_row0_v + (uint64_t)in_page * ROW_BYTES + chunk_in_row * 16;
-                tile.v[i] = *reinterpret_cast<const uint4*>(source);
+                tile.v[i] = load_streaming(source);
             }
         }
     };

@@ -60,11 +60,20 @@ constexpr bool tile_layout_is_linear(int head_dim, bool fp8_pages) { return (hea
 // lds_address + 16 * l (lds_address is wave-uniform and travels in M0).  Written as inline assembly on purpose: the
 // compiler makes every LDS read wait for all direct-to-LDS loads it knows of (it cannot tell which tile a read
 // touches), which would allow only one tile in flight; here the waits are explicit (wait_vmem_outstanding).
+// STREAMING marks bytes that no other block of the launch reads again (nt: they take no room in this XCD's L2).
+template <bool STREAMING>
 __device__ __forceinline__ void load_to_lds_b128(const unsigned char* uniform_base, uint32_t lane_offset, uint32_t lds_address) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :
-                 : "v"(lane_offset), "s"(uniform_base), "s"(lds_address)
-                 : "memory", "m0");
+    if constexpr (STREAMING) {
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt"
+                     :
+                     : "v"(lane_offset), "s"(uniform_base), "s"(lds_address)
+                     : "memory", "m0");
+    } else {
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :
+                     : "v"(lane_offset), "s"(uniform_base), "s"(lds_address)
+                     : "memory", "m0");
+    }
 }
 
 // Byte address of an LDS location as the hardware sees it.
@@ -106,6 +115,10 @@ void tile_map_kernel(const MapParams p) {
     constexpr int SL = BK / 32;                     // slices per tile
     constexpr int PAGE_ROW = D * (KV8 ? 1 : 2);     // bytes of one K/V row in a page
     constexpr int CPR = PAGE_ROW / 16;              // 16-byte chunks per K/V row in a page
+    // The verify tiles (one column tile per wave, four waves: one block per KV range and KV head of a speculative block) are
+    // the only readers of their K/V bytes, which therefore stream; the Q tiles of a prefill chunk share theirs through
+    // the XCD's L2 (streaming loads there: 4.27 -> 4.40 ms).
+    constexpr bool STREAM_KV = NTW == 1 && NWAVES == 4;
     constexpr bool LINEAR = tile_layout_is_linear(D, KV8);
     constexpr bool LINEAR_LOADS = LINEAR && !KV8;   // direct-to-LDS loads that fill the linear layout's units themselves
     constexpr int HALVES = LINEAR_LOADS ? D / 128 : 1;    // ... wave loads per row group (each takes 128 dims of four rows)
@@ -393,7 +406,7 @@ void tile_map_kernel(const MapParams p) {
         if (tile_token >= blk_lo && tile_token + BK <= blk_hi) {
 #pragma unroll
             for (int j = 0; j < LPW; ++j)
-                load_to_lds_b128(k_plane_base + (uint64_t)ids[load_id(j)] * p.page_bytes, lane_offset[j], load_lds_address(j, stage));
+                load_to_lds_b128<STREAM_KV>(k_plane_base + (uint64_t)ids[load_id(j)] * p.page_bytes, lane_offset[j], load_lds_address(j, stage));
             return;
         }
         // first or last tile of the range: rows outside it are redirected, which changes their offsets
@@ -404,7 +417,7 @@ void tile_map_kernel(const MapParams p) {
             token = token < blk_lo ? blk_lo : token;
             token = token >= blk_hi ? blk_hi - 1 : token;
             const uint32_t offset = (token & (tpp - 1)) * PAGE_ROW + (source.chunk << 4) + (load_is_v(j) ? v_plane_distance : 0u);
-            load_to_lds_b128(k_plane_base + (uint64_t)ids[load_id(j)] * p.page_bytes, offset, load_lds_address(j, stage));
+            load_to_lds_b128<STREAM_KV>(k_plane_base + (uint64_t)ids[load_id(j)] * p.page_bytes, offset, load_lds_address(j, stage));
         }
     };
 
@@ -423,7 +436,7 @@ void tile_map_kernel(const MapParams p) {
     auto issue_interior_tile = [&](uint32_t stage, const TileIds ids) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < LPW; ++j)
-            load_to_lds_b128(k_plane_base + (uint64_t)ids[load_id(j)] * p.page_bytes, lane_offset[j], load_lds_address(j, stage));
+            load_to_lds_b128<STREAM_KV>(k_plane_base + (uint64_t)ids[load_id(j)] * p.page_bytes, lane_offset[j], load_lds_address(j, stage));
     };
 
     // FP8 pages: one tile in registers, decoded into the bf16 LDS layout the direct loads would have produced
