@@ -31,8 +31,8 @@ NUM_POOLS = 3
 # HBM bytes per Map launch from the hardware counters, (FETCH_SIZE * 2.000 + WRITE_SIZE * 1.000) KiB per dispatch:
 # two `rocprofv3 --pmc` runs per config, each counter scaled by what it reads for a plain 1 GiB copy kernel
 # (`--calibration-copy`).  The summaries with their commands are the text files under profiles/.
-MEASURED_MAP_TRAFFIC_BYTES = {2: 564_434_944, 3: 2_151_780_352, 4: 1_447_223_296, 5: 1_202_804_736, 6: 1_068_930_048}
-MEASURED_MAP_TRAFFIC_BYTES_FP8_PAGES = {2: 285_208_576, 3: 1_077_938_176, 4: 729_363_456, 5: 869_689_344, 6: 1_614_070_784}
+MEASURED_MAP_TRAFFIC_BYTES = {2: 565_561_344, 3: 2_153_930_752, 4: 1_446_890_496, 5: 1_202_827_264, 6: 1_068_915_712}
+MEASURED_MAP_TRAFFIC_BYTES_FP8_PAGES = {2: 286_631_936, 3: 1_082_411_008, 4: 729_135_104, 5: 869_629_952, 6: 1_614_041_088}
 
 CONFIGS = {
     1: dict(name="config1: B=1 q=1 Hq32/Hkv8/D128 ctx 1024, identity pages", hq=32, hkv=8, d=128, kind="decode", kv_slice=64),

@@ -88,10 +88,11 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
 
-// Streaming accesses (nt): bytes that are written once for a later launch, or read once by this block and by no other.
-// They take no room in the XCD's L2 from data that is used again.  Measured on the decode Map: 107 -> 98 us on a
-// 32-request batch; on the verify tiles 240 -> 223 us; on RMSNorm + RoPE rows 102 -> 86 us with streaming stores (and
-// 94 us with streaming loads as well, so its loads stay ordinary ones).
+// Streaming accesses (the nt bit of the memory instruction: a hint that the bytes will not be used again soon), for bytes
+// that are written once for a later launch, or read once by this block and by no other.  Measured: decode Map 107 -> 98 us
+// on a 32-request batch and verify tiles 240 -> 223 us with streaming K/V loads, at unchanged HBM traffic; RMSNorm + RoPE
+// rows 102 -> 86 us with streaming stores (94 us with streaming loads as well, so its loads stay ordinary ones); K/V tiles
+// that several blocks share through the L2 (prefill) lose with the hint and do not get it.
 __device__ __forceinline__ void store_streaming(void* target, uint4 value) {
     typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
     const U32x4 v = {value.x, value.y, value.z, value.w};

@@ -60,7 +60,7 @@ constexpr bool tile_layout_is_linear(int head_dim, bool fp8_pages) { return (hea
 // lds_address + 16 * l (lds_address is wave-uniform and travels in M0).  Written as inline assembly on purpose: the
 // compiler makes every LDS read wait for all direct-to-LDS loads it knows of (it cannot tell which tile a read
 // touches), which would allow only one tile in flight; here the waits are explicit (wait_vmem_outstanding).
-// STREAMING marks bytes that no other block of the launch reads again (nt: they take no room in this XCD's L2).
+// STREAMING marks bytes that no other block of the launch reads again (the nt bit: a hint not to keep them cached).
 template <bool STREAMING>
 __device__ __forceinline__ void load_to_lds_b128(const unsigned char* uniform_base, uint32_t lane_offset, uint32_t lds_address) {
     if constexpr (STREAMING) {
