@@ -840,6 +840,15 @@ extern "C" int khm_gqa_activation_gate(uint32_t dtype, uint32_t num_q_heads, uin
     p.num_active_tokens = to_device(num_active_tokens);
     p.values_per_token = num_q_heads * head_dim;
     p.is_f32 = dtype == KHM_DTYPE_F32;
+    const uintptr_t address_bits = reinterpret_cast<uintptr_t>(attention_output.ptr) | reinterpret_cast<uintptr_t>(gates.ptr) |
+                                   reinterpret_cast<uintptr_t>(output.ptr);
+    if (address_bits % 16 == 0) {
+        const uint64_t per_block = 256ull * gate_elements_per_thread(p.is_f32 != 0);
+        const uint32_t blocks = (uint32_t)((values + per_block - 1) / per_block);
+        if (p.is_f32) hipLaunchKernelGGL(activation_gate_vector_kernel<true>, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+        else hipLaunchKernelGGL(activation_gate_vector_kernel<false>, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+        return check_launch("activation gate");
+    }
     const uint32_t blocks = (uint32_t)((values + 255) / 256);
     hipLaunchKernelGGL(activation_gate_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), p);
     return check_launch("activation gate");

@@ -103,6 +103,11 @@ __device__ __forceinline__ void store_streaming(void* target, uint2 value) {
     const U32x2 v = {value.x, value.y};
     __builtin_nontemporal_store(v, reinterpret_cast<U32x2*>(target));
 }
+__device__ __forceinline__ void store_streaming(void* target, float4 value) {
+    typedef float F32x4 __attribute__((ext_vector_type(4)));
+    const F32x4 v = {value.x, value.y, value.z, value.w};
+    __builtin_nontemporal_store(v, reinterpret_cast<F32x4*>(target));
+}
 __device__ __forceinline__ uint4 load_streaming(const void* source) {
     typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
     const U32x4 v = __builtin_nontemporal_load(reinterpret_cast<const U32x4*>(source));
@@ -133,12 +138,14 @@ __device__ __forceinline__ float coherent_load_f32(const float* address) {
 __device__ __forceinline__ float round_to_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
 
 // gqa_activation_gate.metal:19-26: sigmoid with every step rounded to bf16.
+// `x` is a decoded bf16 value (every caller passes one), so |x| and -|x| are bf16 values already and their rounding steps
+// are identities; the denominator is one of the 129 bf16 values in [1, 2], for each of which v_rcp_f32 rounds to the same
+// bf16 as the exact quotient (checked, with everything else, over all 65 536 gate patterns against the oracle).
 __device__ __forceinline__ float sigmoid_bf16_steps(float x) {
-    const float abs_x = round_to_bf16(fabsf(x));
-    const float neg_abs_x = round_to_bf16(-abs_x);
+    const float neg_abs_x = -fabsf(x);
     const float exp_x = round_to_bf16(__expf(neg_abs_x));
     const float denom = round_to_bf16(1.0f + exp_x);
-    const float y = round_to_bf16(1.0f / denom);
+    const float y = round_to_bf16(__builtin_amdgcn_rcpf(denom));
     return x < 0.0f ? round_to_bf16(1.0f - y) : y;
 }
 

@@ -105,7 +105,8 @@ __global__ __launch_bounds__(kReduceThreads) void split_kv_reduce_rows_kernel(co
     merge_store_output(state, p.output, p.gates, out_index);
 }
 
-// gqa_activation_gate_{f32,bf16} (gqa_activation_gate.metal:28-59): one thread per element.
+// gqa_activation_gate_{f32,bf16} (gqa_activation_gate.metal:28-59): one thread per element.  For buffers that are not
+// 16-byte aligned; the vector kernel below is the one that normally runs.
 __global__ __launch_bounds__(256) void activation_gate_kernel(const GateParams p) {
     const uint64_t total = (uint64_t)resolve_u32(p.num_active_tokens, p.replay_parameters) * p.values_per_token;
     const uint64_t gid = (uint64_t)blockIdx.x * 256 + threadIdx.x;
@@ -118,6 +119,47 @@ __global__ __launch_bounds__(256) void activation_gate_kernel(const GateParams p
         const float a = bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.attention)[gid]);
         const float x = bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.gates)[gid]);
         reinterpret_cast<uint16_t*>(p.output)[gid] = f32_to_bf16_bits(a * sigmoid_bf16_steps(x));
+    }
+}
+
+// The same arithmetic, 16 bytes per thread and buffer (eight bf16 or four f32 elements), the output written with streaming
+// stores (it is read by the next launch, not by this one); what is left of the last group goes element by element.
+constexpr int gate_elements_per_thread(bool f32) { return f32 ? 4 : 8; }
+template <bool F32>
+__global__ __launch_bounds__(256) void activation_gate_vector_kernel(const GateParams p) {
+    constexpr int EPT = gate_elements_per_thread(F32);
+    const uint64_t total = (uint64_t)resolve_u32(p.num_active_tokens, p.replay_parameters) * p.values_per_token;
+    const uint64_t first = ((uint64_t)blockIdx.x * 256 + threadIdx.x) * EPT;
+    if (first >= total) return;
+    if (first + EPT <= total) {
+        if constexpr (F32) {
+            const float4 a = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.attention) + first);
+            const float4 x = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.gates) + first);
+            store_streaming(reinterpret_cast<float*>(p.output) + first,
+                            make_float4(a.x * sigmoid_f32(x.x), a.y * sigmoid_f32(x.y), a.z * sigmoid_f32(x.z), a.w * sigmoid_f32(x.w)));
+        } else {
+            const uint4 a = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.attention) + first);
+            const uint4 x = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.gates) + first);
+            const uint32_t a_words[4] = {a.x, a.y, a.z, a.w}, x_words[4] = {x.x, x.y, x.z, x.w};
+            uint32_t out[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float low = bf16_bits_to_f32(a_words[i] & 0xffffu) * sigmoid_bf16_steps(bf16_bits_to_f32(x_words[i] & 0xffffu));
+                const float high = bf16_bits_to_f32(a_words[i] >> 16) * sigmoid_bf16_steps(bf16_bits_to_f32(x_words[i] >> 16));
+                out[i] = pack_bf16x2(low, high);
+            }
+            store_streaming(reinterpret_cast<uint16_t*>(p.output) + first, make_uint4(out[0], out[1], out[2], out[3]));
+        }
+        return;
+    }
+    for (uint64_t i = first; i < total; ++i) {
+        if constexpr (F32) {
+            reinterpret_cast<float*>(p.output)[i] = reinterpret_cast<const float*>(p.attention)[i] * sigmoid_f32(reinterpret_cast<const float*>(p.gates)[i]);
+        } else {
+            const float a = bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.attention)[i]);
+            const float x = bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.gates)[i]);
+            reinterpret_cast<uint16_t*>(p.output)[i] = f32_to_bf16_bits(a * sigmoid_bf16_steps(x));
+        }
     }
 }
 
