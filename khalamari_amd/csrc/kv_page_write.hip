@@ -17,50 +17,76 @@
 namespace khm {
 
 
-// A block serves one token write (blockIdx.x), so the request slot, the page-table walk and the page address are
-// wave-uniform scalar work; a thread moves eight consecutive dims of one KV head's row, for K and for V: a 16-byte load
-// each, then a 16-byte (bf16 pages) or 8-byte (FP8 pages) store each.  Head dims that are no multiple of eight take the
-// scalar tail.
+// A block serves kWritesPerBlock consecutive token writes; a thread moves eight consecutive dims of one KV head's row for
+// each of them, for K and for V: a 16-byte load each, then a 16-byte (bf16 pages) or 8-byte (FP8 pages) streaming store
+// each.  The request slots, positions, page ids and rows of all of a block's writes are requested before the first is
+// used, so the chain slot/position -> page id -> store is walked for four tokens at once (16384 writes of 8 heads x 128
+// dims into FP8 pages: 18.7 us; 20.8 us with one write per block and the walk as scalar work, 20.4 / 22.2 us with eight /
+// sixteen writes per block).  Head dims that are no multiple of eight take the scalar tail.
+constexpr int kWritesPerBlock = 4;
 template <bool FP8_PAGES>
 __global__ __launch_bounds__(1024) void kv_page_write_kernel(const PageWriteParams p) {
-    const uint32_t write_index = blockIdx.x;
-    if (write_index >= resolve_u32(p.num_active_token_writes, p.replay_parameters)) return;
+    const uint32_t num_active = resolve_u32(p.num_active_token_writes, p.replay_parameters);
+    const uint32_t first_write = blockIdx.x * kWritesPerBlock;
+    if (first_write >= num_active) return;
     const uint32_t chunks_per_row = (p.head_dim + 7) / 8;
     const uint32_t in_write = blockIdx.y * blockDim.x + threadIdx.x;
     if (in_write >= p.num_kv_heads * chunks_per_row) return;
     const uint32_t head = in_write / chunks_per_row;
     const uint32_t dim = (in_write - head * chunks_per_row) * 8;
-
-    const uint32_t req_slot = p.req_slots[write_index];
-    const uint32_t token = p.flat_token_indices[write_index];
     const uint32_t layer = resolve_u32(p.layer_index, p.replay_parameters);
     constexpr uint32_t kElementBytes = FP8_PAGES ? 1 : 2;
-    const PageTarget target = page_target_of(p, req_slot, token, layer, head, dim, kElementBytes);
-    uint8_t* k_target = p.pages + target.k_offset;
-    uint8_t* v_target = k_target + target.v_distance;
-    const uint64_t source = ((uint64_t)write_index * p.num_kv_heads + head) * p.head_dim + dim;
 
-    if (dim + 8 <= p.head_dim && p.head_dim % 8 == 0) {
-        const uint4 k = *reinterpret_cast<const uint4*>(p.flat_k + source);
-        const uint4 v = *reinterpret_cast<const uint4*>(p.flat_v + source);
-        if constexpr (FP8_PAGES) {
-            auto encode8 = [](uint4 bits) { return bf16x8_bits_to_fp8x8_e4m3fn(bits); };
-            store_streaming(k_target, encode8(k));
-            store_streaming(v_target, encode8(v));
-        } else {
-            store_streaming(k_target, k);
-            store_streaming(v_target, v);
+    bool live[kWritesPerBlock];
+    uint32_t write_index[kWritesPerBlock], req_slot[kWritesPerBlock], token[kWritesPerBlock];
+#pragma unroll
+    for (int w = 0; w < kWritesPerBlock; ++w) {
+        live[w] = first_write + w < num_active;
+        write_index[w] = live[w] ? first_write + w : first_write;
+        req_slot[w] = p.req_slots[write_index[w]];
+        token[w] = p.flat_token_indices[write_index[w]];
+    }
+    if (p.head_dim % 8 == 0) {
+        uint4 k[kWritesPerBlock], v[kWritesPerBlock];
+        PageTarget target[kWritesPerBlock];
+#pragma unroll
+        for (int w = 0; w < kWritesPerBlock; ++w) {
+            const uint64_t source = ((uint64_t)write_index[w] * p.num_kv_heads + head) * p.head_dim + dim;
+            k[w] = *reinterpret_cast<const uint4*>(p.flat_k + source);
+            v[w] = *reinterpret_cast<const uint4*>(p.flat_v + source);
+            target[w] = page_target_of(p, req_slot[w], token[w], layer, head, dim, kElementBytes);
+        }
+#pragma unroll
+        for (int w = 0; w < kWritesPerBlock; ++w) {
+            if (!live[w]) continue;
+            uint8_t* k_target = p.pages + target[w].k_offset;
+            uint8_t* v_target = k_target + target[w].v_distance;
+            if constexpr (FP8_PAGES) {
+                store_streaming(k_target, bf16x8_bits_to_fp8x8_e4m3fn(k[w]));
+                store_streaming(v_target, bf16x8_bits_to_fp8x8_e4m3fn(v[w]));
+            } else {
+                store_streaming(k_target, k[w]);
+                store_streaming(v_target, v[w]);
+            }
         }
         return;
     }
-    for (uint32_t i = 0; i < 8 && dim + i < p.head_dim; ++i) {
-        const uint32_t k = p.flat_k[source + i], v = p.flat_v[source + i];
-        if constexpr (FP8_PAGES) {
-            k_target[i] = (uint8_t)bf16_bits_to_fp8_e4m3fn(k);
-            v_target[i] = (uint8_t)bf16_bits_to_fp8_e4m3fn(v);
-        } else {
-            reinterpret_cast<uint16_t*>(k_target)[i] = (uint16_t)k;
-            reinterpret_cast<uint16_t*>(v_target)[i] = (uint16_t)v;
+#pragma unroll
+    for (int w = 0; w < kWritesPerBlock; ++w) {
+        if (!live[w]) continue;
+        const PageTarget target = page_target_of(p, req_slot[w], token[w], layer, head, dim, kElementBytes);
+        uint8_t* k_target = p.pages + target.k_offset;
+        uint8_t* v_target = k_target + target.v_distance;
+        const uint64_t source = ((uint64_t)write_index[w] * p.num_kv_heads + head) * p.head_dim + dim;
+        for (uint32_t i = 0; i < 8 && dim + i < p.head_dim; ++i) {
+            const uint32_t k = p.flat_k[source + i], v = p.flat_v[source + i];
+            if constexpr (FP8_PAGES) {
+                k_target[i] = (uint8_t)bf16_bits_to_fp8_e4m3fn(k);
+                v_target[i] = (uint8_t)bf16_bits_to_fp8_e4m3fn(v);
+            } else {
+                reinterpret_cast<uint16_t*>(k_target)[i] = (uint16_t)k;
+                reinterpret_cast<uint16_t*>(v_target)[i] = (uint16_t)v;
+            }
         }
     }
 }
@@ -196,7 +222,7 @@ extern "C" int khm_kv_page_write(const khm_kv_page_write_config* config, const k
     const uint32_t block_threads = (uint32_t)(chunks_per_write >= 1024 ? 1024 : (chunks_per_write + 63) / 64 * 64);
     const uint64_t chunk_blocks = (chunks_per_write + block_threads - 1) / block_threads;
     KHM_REQUIRE(chunk_blocks <= 65535, "GQA KV page write: %llu chunks per token write exceed the launch grid", (unsigned long long)chunks_per_write);
-    const dim3 grid(shape->num_total_token_writes, (uint32_t)chunk_blocks);
+    const dim3 grid((shape->num_total_token_writes + kWritesPerBlock - 1) / kWritesPerBlock, (uint32_t)chunk_blocks);
     if (config->kv_dtype == KHM_DTYPE_FP8_E4M3FN) {
         hipLaunchKernelGGL(kv_page_write_kernel<true>, grid, dim3(block_threads), 0, static_cast<hipStream_t>(stream), p);
     } else {
