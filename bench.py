@@ -201,6 +201,9 @@ class Workload:
         partial_dtype = DTYPE_F32 if os.environ.get("KHM_BENCH_PARTIAL", "bf16") == "f32" else DTYPE_BF16
         fixed = ReplayU32.fixed
         md = self.metadata
+        # The launch closures hold these tensors, not the workload: a closure over `self` stored on `self` is a reference
+        # cycle, and a workload in a cycle keeps its device memory until the cycle collector runs, whenever that is.
+        q, page_table, out, gates = self.q, self.page_table, self.out, self.gates
         # Map and Reduce in one launch (the last block of a token merges) pays off when the step is launch-latency
         # bound; large batches keep the two-launch form.  KHM_BENCH_FUSED=0/1 forces either.
         choice = os.environ.get("KHM_BENCH_FUSED", "auto")
@@ -215,7 +218,7 @@ class Workload:
             self._keep = (compute, scratch)
 
             def launch_map(pool):
-                compute.invoke_map(q=self.q, kv_pages=pool, req_slots=md.req_slots(), page_ids=self.page_table,
+                compute.invoke_map(q=q, kv_pages=pool, req_slots=md.req_slots(), page_ids=page_table,
                                    sdpa_map_task_templates=md.sdpa_map_task_templates(), partial_exp_sums=scratch.partial_exp_sums,
                                    partial_max_logits=scratch.partial_max_logits, partial_output=scratch.partial_output,
                                    page_table_index=fixed(0), num_active_tokens=fixed(shape.num_tokens),
@@ -224,27 +227,27 @@ class Workload:
             def launch_reduce():
                 compute.invoke_reduce(partial_exp_sums=scratch.partial_exp_sums, partial_max_logits=scratch.partial_max_logits,
                                       partial_output=scratch.partial_output, cu_sdpa_partial_outputs=md.cu_sdpa_partial_outputs(),
-                                      output=self.out, num_active_tokens=fixed(shape.num_tokens), gates=self.gates)
+                                      output=out, num_active_tokens=fixed(shape.num_tokens), gates=gates)
 
             if fused:
                 counters = torch.zeros(compute.arrival_counters_bytes(), dtype=torch.uint8, device=device)
                 self._keep += (counters,)
 
                 def launch_map(pool):  # noqa: F811
-                    compute.invoke_map_reduce(q=self.q, kv_pages=pool, req_slots=md.req_slots(), page_ids=self.page_table,
+                    compute.invoke_map_reduce(q=q, kv_pages=pool, req_slots=md.req_slots(), page_ids=page_table,
                                               sdpa_map_task_templates=md.sdpa_map_task_templates(),
                                               partial_exp_sums=scratch.partial_exp_sums, partial_max_logits=scratch.partial_max_logits,
                                               partial_output=scratch.partial_output,
-                                              cu_sdpa_partial_outputs=md.cu_sdpa_partial_outputs(), output=self.out,
+                                              cu_sdpa_partial_outputs=md.cu_sdpa_partial_outputs(), output=out,
                                               arrival_counters=counters, page_table_index=fixed(0),
                                               num_active_tokens=fixed(shape.num_tokens),
-                                              num_active_kv_splits=fixed(shape.num_sdpa_map_task_templates), gates=self.gates)
+                                              num_active_kv_splits=fixed(shape.num_sdpa_map_task_templates), gates=gates)
 
                 launch_reduce = None
         else:
             config = sliced_q.Config(hq, hkv, d, d ** -0.5, self.page_bytes, layout, DTYPE_BF16, kv_dtype, partial_dtype)
             qshape = sliced_q.Shape(shape.num_total_tokens, shape.num_total_q_token_tiles, shape.num_total_sdpa_map_task_templates)
-            common = dict(q=self.q, req_slots=md.req_slots(), page_ids=self.page_table,
+            common = dict(q=q, req_slots=md.req_slots(), page_ids=page_table,
                           visible_kv_token_ranges=md.visible_kv_token_ranges(), q_token_ranges=md.q_token_ranges(),
                           sdpa_map_task_templates=md.sdpa_map_task_templates(), page_table_index=fixed(0),
                           num_active_tokens=fixed(shape.num_tokens), num_active_q_token_tiles=fixed(shape.num_q_token_tiles))
@@ -253,7 +256,7 @@ class Workload:
                 self._keep = (compute,)
 
                 def launch_map(pool):
-                    compute.invoke_direct(kv_pages=pool, output=self.out, **common)
+                    compute.invoke_direct(kv_pages=pool, output=out, **common)
 
                 launch_reduce = None
             else:
@@ -270,7 +273,7 @@ class Workload:
                 def launch_reduce():
                     compute.invoke_reduce(partial_output=partial, partial_exp_sums=sums, partial_max_logits=maxs,
                                           q_token_ranges=md.q_token_ranges(), cu_sdpa_partial_outputs=md.cu_sdpa_partial_outputs(),
-                                          output=self.out, num_active_q_token_tiles=fixed(shape.num_q_token_tiles))
+                                          output=out, num_active_q_token_tiles=fixed(shape.num_q_token_tiles))
 
                 if fused:
                     counters = torch.zeros(compute.arrival_counters_bytes(), dtype=torch.uint8, device=device)
@@ -278,7 +281,7 @@ class Workload:
 
                     def launch_map(pool):  # noqa: F811
                         compute.invoke_map_reduce(kv_pages=pool, partial_output=partial, partial_exp_sums=sums, partial_max_logits=maxs,
-                                                  cu_sdpa_partial_outputs=md.cu_sdpa_partial_outputs(), output=self.out,
+                                                  cu_sdpa_partial_outputs=md.cu_sdpa_partial_outputs(), output=out,
                                                   arrival_counters=counters,
                                                   num_active_kv_splits=fixed(shape.num_sdpa_map_task_templates), **common)
 

@@ -626,7 +626,10 @@ int khm_selection_cu_partial_outputs(const khm_selection* selection, uint32_t* o
 /* GQAMetadataBuffers (attn/gqa/batch_metadata.rs:98-326): capacity-sized device arrays refreshed from one
  * selection.  update() fills pinned staging memory and enqueues the host-to-device copies on `stream`
  * (the reference writes shared-memory buffers directly); arrays the reference leaves untouched stay
- * untouched (q_token_ranges for the sliced-KV kind, every tail beyond the written prefix). */
+ * untouched (q_token_ranges for the sliced-KV kind, every tail beyond the written prefix).
+ * create() and destroy() allocate and free device and pinned memory, and update() waits for `stream`: none of the three
+ * may run while any stream of the process is under hipGraph capture in the global mode (the capture is invalidated and
+ * its next enqueue fails).  A host language with finalizers must not leave destroy() to its collector. */
 typedef struct khm_gqa_metadata khm_gqa_metadata;
 typedef enum khm_gqa_metadata_array {
     KHM_METADATA_REQ_SLOTS = 0,               /* u32 [max_tokens] */

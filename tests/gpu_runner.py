@@ -1,6 +1,8 @@
 """Runs a Workload through the C ABI on the GPU (torch provides device memory and the stream only)."""
 from __future__ import annotations
 
+import gc
+
 import numpy as np
 import torch
 
@@ -17,6 +19,24 @@ def to_device(array: np.ndarray, device) -> torch.Tensor:
     if array.dtype == np.uint32:
         return torch.from_numpy(array.view(np.int32)).to(device)
     return torch.from_numpy(array).to(device)
+
+
+def capture_graph(record) -> torch.cuda.CUDAGraph:
+    """`record()` captured into a HIP graph.  A capture is invalidated by any call that frees or allocates device or pinned
+    memory in the process while it is open, and Python runs finalizers of dead reference cycles (a metadata buffer set's
+    hipFree, say) whenever its cycle collector fires: collect first, and keep the collector off until the capture ends."""
+    gc.collect()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    collector_was_on = gc.isenabled()
+    gc.disable()
+    try:
+        with torch.cuda.graph(graph):
+            record()
+    finally:
+        if collector_was_on:
+            gc.enable()
+    return graph
 
 
 def bf16_tensor_to_f32(t: torch.Tensor) -> np.ndarray:

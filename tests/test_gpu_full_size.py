@@ -106,3 +106,23 @@ def test_partitioning_does_not_change_the_result_at_full_size(device):
         torch.cuda.empty_cache()
     for other in results[1:]:
         helpers.assert_parity(other, results[0], "partition invariance")
+
+
+@pytest.mark.parametrize("index", [1, 2, 4, 5])
+def test_workload_is_released_without_the_cycle_collector(device, index):
+    """A workload dropped by its owner gives back its pools and its metadata buffers (hipFree, hipHostFree) at once, by
+    reference count.  Left to the cycle collector it would hold tens of gigabytes until some later allocation count is
+    reached, and its frees could land inside another test's graph capture, which they would invalidate."""
+    import gc
+    import weakref
+
+    gc.collect()
+    gc.disable()
+    try:
+        workload = bench.Workload(index, device, num_pools=1)
+        _run_step(workload)
+        alive = [weakref.ref(workload), weakref.ref(workload.metadata), weakref.ref(workload.launch_map)]
+        del workload
+        assert [ref() for ref in alive] == [None, None, None]
+    finally:
+        gc.enable()

@@ -49,10 +49,7 @@ def test_decode_program_replays_with_different_active_counts(device):
 
     params.copy_(arguments(tokens))
     record()                       # eager warm-up before capture
-    torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        record()
+    graph = gpu_runner.capture_graph(record)
     for active in [tokens, 1, 5, 3, 8, 2]:
         print(f"graph replay active={active}", flush=True)
         out.fill_(POISON)          # a fill kernel, eager, between replays
@@ -105,10 +102,7 @@ def test_verify_program_replays_on_the_tiled_kernel(device):
 
     params.copy_(arguments(len(q_lens))[1])
     record()
-    torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        record()
+    graph = gpu_runner.capture_graph(record)
     for active_requests in [4, 1, 3, 2, 4]:
         active_tokens, block = arguments(active_requests)
         print(f"verify graph replay requests={active_requests}", flush=True)

@@ -116,9 +116,7 @@ def test_static_scratch_call_under_graph_capture_allocates_nothing(device):
     free_after, _ = torch.cuda.mem_get_info(device)
     assert free_after == free_before and torch.cuda.memory_allocated(device) == allocated_before
 
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        compute.invoke_map_reduce_static(output=out, **common)
+    graph = gpu_runner.capture_graph(lambda: compute.invoke_map_reduce_static(output=out, **common))
     for replay in range(3):
         print(f"static scratch graph replay {replay}", flush=True)
         out.fill_(0x4228)           # eager fill kernel between the replays
