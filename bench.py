@@ -470,8 +470,8 @@ def cpu_baseline(index: int = 2, seconds_hint: float = 20.0) -> dict:
 
 
 def producer_rows(device, steps: int = 20) -> dict:
-    """The kernels that feed the SDPA, at config 5's prefill shape (8 x 2048 new tokens, Hq=64 / Hkv=8, D=128): per-head
-    RMSNorm + RoPE of Q, the K/V page write into FP8 pages, and K RMSNorm + RoPE fused with that write.  All are HBM bound;
+    """The kernels that feed the SDPA, at config 5's prefill shape (8 x 2048 new tokens, Hq=64 / Hkv=8, D=128): the split of
+    the gated input projection, per-head RMSNorm + RoPE of Q, the K/V page write into FP8 pages, and K RMSNorm + RoPE fused with that write.  All are HBM bound;
     bytes are what the kernel must move."""
     import torch
 
@@ -498,6 +498,21 @@ def producer_rows(device, steps: int = 20) -> dict:
         return float(np.mean([a.elapsed_time(b) for a, b in pairs])) * 1e3
 
     result = {}
+    from khalamari_amd import qgkv_split
+
+    split_config = qgkv_split.Config.bf16(hq, hkv, d)
+    split_shape = qgkv_split.Shape(tokens)
+    projection = torch.randn((tokens, split_config.projection_width()), device=device, dtype=torch.bfloat16, generator=generator)
+    split_q, split_g = (torch.empty((tokens, hq, d), device=device, dtype=torch.bfloat16) for _ in range(2))
+    split_k, split_v = (torch.empty((tokens, hkv, d), device=device, dtype=torch.bfloat16) for _ in range(2))
+    split = qgkv_split.Compute(split_config)
+    us = timed(lambda: split.invoke(split_shape, qgkv=projection, q=split_q, g=split_g, k=split_k, v=split_v,
+                                    num_active_tokens=ReplayU32.fixed(tokens)))
+    nbytes = 2 * split_config.projection_bytes(split_shape)
+    result["qgkv_split"] = {"workload": f"projection rows {tokens}x(2x{hq}+2x{hkv})x{d} bf16 -> q, g, k, v", "kernel_us": us,
+                            "algorithmic_bytes": nbytes, "gbps": nbytes / us / 1e3, "roofline_frac": nbytes / us / 1e3 / HBM_PEAK_GBPS}
+    del projection, split_q, split_g, split_k, split_v
+
     q = torch.randn((tokens, hq, d), device=device, dtype=torch.float32, generator=generator).to(torch.bfloat16)
     q_out = torch.empty_like(q)
     weight = torch.ones(d, device=device, dtype=torch.bfloat16)

@@ -353,6 +353,30 @@ int khm_gqa_activation_gate(uint32_t dtype, uint32_t num_q_heads, uint32_t head_
                             khm_replay_u32 num_active_tokens, const uint32_t* replay_parameters, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Split of the fused input projection, the first launch of the layer (attn/gqa/backend.rs:358-370):
+ * components/gqa/qgkv_split.rs:34-236 with gqa_qgkv_split.metal:5-44 (a token's row is
+ * [Hq x (q head | gate head)][Hkv x k head][Hkv x v head]) and components/gqa/qkv_split.rs with
+ * gqa_qkv_split.metal:5-34 ([Hq x q head][Hkv x k head][Hkv x v head]).  The first num_active_tokens rows go to
+ * q, g [T][Hq][D] and k, v [T][Hkv][D]; rows beyond stay untouched.  dtype F32 or BF16; bit-exact.
+ * Buffers must be aligned to their element size; 16-byte alignment gives the widest copies.
+ * ------------------------------------------------------------------------------------------ */
+typedef struct khm_gqa_projection_split_config {
+    uint32_t num_q_heads;
+    uint32_t num_kv_heads;
+    uint32_t head_dim;
+    uint32_t dtype; /* KHM_DTYPE_F32 or KHM_DTYPE_BF16 */
+} khm_gqa_projection_split_config;
+/* Config::qgkv_width / qkv_width: elements of one token's projection row (0: the head count does not fit u32). */
+uint64_t khm_gqa_qgkv_width(const khm_gqa_projection_split_config* config);
+uint64_t khm_gqa_qkv_width(const khm_gqa_projection_split_config* config);
+int khm_gqa_qgkv_split(const khm_gqa_projection_split_config* config, uint32_t num_total_tokens, khm_buffer qgkv,
+                       khm_buffer q, khm_buffer g, khm_buffer k, khm_buffer v, khm_replay_u32 num_active_tokens,
+                       const uint32_t* replay_parameters, void* stream);
+int khm_gqa_qkv_split(const khm_gqa_projection_split_config* config, uint32_t num_total_tokens, khm_buffer qkv,
+                      khm_buffer q, khm_buffer k, khm_buffer v, khm_replay_u32 num_active_tokens,
+                      const uint32_t* replay_parameters, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * FP8 E4M3FN unit-scale codec, host side: components/gqa/fp8.rs:19-58
  * ------------------------------------------------------------------------------------------ */
 uint8_t khm_bf16_to_fp8_e4m3(uint16_t bf16_bits);

@@ -179,6 +179,12 @@ class KvPageWriteConfig(ctypes.Structure):
     _fields_ = [("num_kv_heads", u32), ("head_dim", u32), ("page_bytes", u32), ("dtype", u32), ("kv_dtype", u32)]
 
 
+class ProjectionSplitConfig(ctypes.Structure):
+    """`qgkv_split::Config` / `qkv_split::Config` (qgkv_split.rs:34-40)."""
+
+    _fields_ = [("num_q_heads", u32), ("num_kv_heads", u32), ("head_dim", u32), ("dtype", u32)]
+
+
 class KvPageWriteShape(ctypes.Structure):
     _fields_ = [("num_total_token_writes", u32), ("page_table_layout", PageTableLayoutStruct)]
 
@@ -249,6 +255,7 @@ EXPORTED_SYMBOLS = (
     "khm_sliced_q_direct_gated", "khm_sliced_q_reduce_gated",
     "khm_sliced_q_arrival_counters_bytes", "khm_sliced_q_map_reduce",
     "khm_gqa_activation_gate",
+    "khm_gqa_qgkv_width", "khm_gqa_qkv_width", "khm_gqa_qgkv_split", "khm_gqa_qkv_split",
     "khm_bf16_to_fp8_e4m3", "khm_fp8_e4m3_to_bf16", "khm_f32_to_bf16", "khm_bf16_to_f32",
     "khm_fp8_e4m3_to_bf16_device", "khm_bf16_to_fp8_e4m3_device",
     "khm_kv_page_write_num_tokens_per_page", "khm_kv_page_write",
@@ -337,6 +344,14 @@ def lib() -> ctypes.CDLL:
                                                  ctypes.c_void_p]
     handle.khm_gqa_activation_gate.argtypes = [u32, u32, u32, u32, Buffer, Buffer, Buffer, ReplayU32, ctypes.c_void_p,
                                                ctypes.c_void_p]
+    handle.khm_gqa_qgkv_width.restype = u64
+    handle.khm_gqa_qgkv_width.argtypes = [ctypes.POINTER(ProjectionSplitConfig)]
+    handle.khm_gqa_qkv_width.restype = u64
+    handle.khm_gqa_qkv_width.argtypes = [ctypes.POINTER(ProjectionSplitConfig)]
+    handle.khm_gqa_qgkv_split.argtypes = [ctypes.POINTER(ProjectionSplitConfig), u32, Buffer, Buffer, Buffer, Buffer, Buffer, ReplayU32,
+                                          ctypes.c_void_p, ctypes.c_void_p]
+    handle.khm_gqa_qkv_split.argtypes = [ctypes.POINTER(ProjectionSplitConfig), u32, Buffer, Buffer, Buffer, Buffer, ReplayU32,
+                                         ctypes.c_void_p, ctypes.c_void_p]
     handle.khm_fp8_e4m3_to_bf16_device.argtypes = [Buffer, Buffer, u64, ctypes.c_void_p]
     handle.khm_bf16_to_fp8_e4m3_device.argtypes = [Buffer, Buffer, u64, ctypes.c_void_p]
     handle.khm_kv_page_write_num_tokens_per_page.restype = u32

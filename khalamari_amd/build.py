@@ -26,6 +26,7 @@ SOURCES = [
     "kv_page_write.hip",
     "bidi_block_sdpa.hip",
     "rms_norm_rope.hip",
+    "projection_split.hip",
 ]
 
 HIPCC_FLAGS = [

@@ -496,6 +496,61 @@ def kv_page_write(pages, flat_k_bits, flat_v_bits, req_slots, flat_token_indices
     return out
 
 
+# ---------------------------------------------------------------- projection split
+
+
+def qgkv_split(qgkv, num_q_heads: int, num_kv_heads: int, head_dim: int, num_active_tokens: int, q, g, k, v):
+    """Restatement of gqa_qgkv_split_impl (components/metal/gqa_qgkv_split.metal:5-44), every thread id at once: element
+    `gid` of the first `num_active_tokens` projection rows goes to q, g, k or v by the shader's own index arithmetic.
+    `q`, `g`, `k`, `v` are the buffers' contents before the launch (flat, any element type); modified copies come back."""
+    source = np.asarray(qgkv).reshape(-1)
+    q, g, k, v = (np.array(a, copy=True).reshape(-1) for a in (q, g, k, v))
+    q_slots = num_q_heads * head_dim
+    kv_slots = num_kv_heads * head_dim
+    token_width = 2 * q_slots + 2 * kv_slots
+    gid = np.arange(num_active_tokens * token_width, dtype=np.int64)
+    token = gid // token_width
+    slot_index = gid - token * token_width
+    values = source[gid]
+    in_qg = slot_index < 2 * q_slots
+    qg_pair = slot_index // (2 * head_dim)
+    in_pair = slot_index - qg_pair * 2 * head_dim
+    target = (token * num_q_heads + qg_pair) * head_dim + (in_pair % head_dim)
+    to_q = in_qg & (in_pair < head_dim)
+    to_g = in_qg & ~(in_pair < head_dim)
+    q[target[to_q]] = values[to_q]
+    g[target[to_g]] = values[to_g]
+    slot_index = slot_index - 2 * q_slots
+    to_k = ~in_qg & (slot_index < kv_slots)
+    k[(token * kv_slots + slot_index)[to_k]] = values[to_k]
+    slot_index = slot_index - kv_slots
+    to_v = ~in_qg & ~to_k
+    v[(token * kv_slots + slot_index)[to_v]] = values[to_v]
+    return q, g, k, v
+
+
+def qkv_split(qkv, num_q_heads: int, num_kv_heads: int, head_dim: int, num_active_tokens: int, q, k, v):
+    """Restatement of gqa_qkv_split_impl (components/metal/gqa_qkv_split.metal:5-34), every thread id at once."""
+    source = np.asarray(qkv).reshape(-1)
+    q, k, v = (np.array(a, copy=True).reshape(-1) for a in (q, k, v))
+    q_slots = num_q_heads * head_dim
+    kv_slots = num_kv_heads * head_dim
+    token_width = q_slots + 2 * kv_slots
+    gid = np.arange(num_active_tokens * token_width, dtype=np.int64)
+    token = gid // token_width
+    slot_index = gid - token * token_width
+    values = source[gid]
+    to_q = slot_index < q_slots
+    q[(token * q_slots + slot_index)[to_q]] = values[to_q]
+    slot_index = slot_index - q_slots
+    to_k = ~to_q & (slot_index < kv_slots)
+    k[(token * kv_slots + slot_index)[to_k]] = values[to_k]
+    slot_index = slot_index - kv_slots
+    to_v = ~to_q & ~to_k
+    v[(token * kv_slots + slot_index)[to_v]] = values[to_v]
+    return q, k, v
+
+
 # ---------------------------------------------------------------- page packing (test helper)
 
 
