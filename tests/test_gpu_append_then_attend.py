@@ -111,3 +111,82 @@ def test_norm_rope_page_write_then_attend_on_one_stream(device, fp8_pages, hq, h
     helpers.assert_parity(actual, expected_from_device, "attention over the rows the producers just wrote")
     # and the whole chain against the oracle's chain, where a moved bf16 rounding in Q or K shows as a slightly different score
     helpers.assert_parity(actual, expected, "norm + rope, page write, attention on one stream", abs_tol=4e-3)
+
+
+@pytest.mark.parametrize("fp8_pages", [True, False])
+@pytest.mark.parametrize("hq,hkv,d,tile", [(16, 2, 128, 32), (12, 2, 256, 8)])
+def test_layer_from_the_projection_rows_to_the_gated_output_on_one_stream(device, fp8_pages, hq, hkv, d, tile):
+    """Everything GQA::record enqueues between the input and the output projection (backend.rs:358-421), five launches on
+    one stream with no host synchronisation: the split of the gated projection rows into q, g, k, v, Q norm + RoPE, the
+    fused K norm + RoPE + K/V page write, and the SDPA with the sigmoid gate applied where the output is written."""
+    from khalamari_amd import qgkv_split
+
+    histories, q_lens = [300, 0, 1000, 77], [40, 17, 5, 1]
+    tpp = 16
+    w = helpers.make_workload(num_q_heads=hq, num_kv_heads=hkv, head_dim=d, tokens_per_page=tpp, histories=histories, q_lens=q_lens,
+                              seed=950 + d + tile, fp8_pages=fp8_pages, garbage_bits=(0x7F if fp8_pages else 0x7FC0))
+    g = w.geom
+    rng = np.random.default_rng(951)
+    total = w.num_tokens
+    bits = lambda shape, scale: oracle.f32_to_bf16_bits((rng.standard_normal(shape) * scale).astype(np.float32))  # noqa: E731
+    q_raw, gate_bits = bits((total, hq, d), 2.0), bits((total, hq, d), 1.5)
+    k_raw, v_new = bits((total, hkv, d), 2.0), bits((total, hkv, d), 1.0)
+    # a projection row: [Hq x (q head | gate head)][Hkv x k head][Hkv x v head] (gqa_qgkv_split.metal:24-43)
+    projection = np.concatenate([np.stack([q_raw, gate_bits], axis=2).reshape(total, 2 * hq * d), k_raw.reshape(total, -1),
+                                 v_new.reshape(total, -1)], axis=1)
+    weight_q = oracle.f32_to_bf16_bits((0.75 + rng.random(d) * 0.5).astype(np.float32))
+    weight_k = oracle.f32_to_bf16_bits((0.75 + rng.random(d) * 0.5).astype(np.float32))
+    positions = np.concatenate([h + np.arange(n) for h, n in zip(histories, q_lens)]).astype(np.uint32)
+
+    to = lambda a: gpu_runner.to_device(np.ascontiguousarray(a), device)  # noqa: E731
+    pages = to(w.kv_pages)
+    positions_d, slots_d, table_d = to(positions), to(w.req_slots), to(w.page_ids)
+    rows = lambda heads: torch.full((total, heads, d), 0x4228, dtype=torch.int16, device=device)  # noqa: E731
+    q_split, g_split, k_split, v_split, q_rows, out = rows(hq), rows(hq), rows(hkv), rows(hkv), rows(hq), rows(hq)
+    norm_q = rnr.Config.bf16(hq, d, d, EPS, THETA).with_norm_weight_dtype(DTYPE_BF16)
+    norm_k = rnr.Config.bf16(hkv, d, d, EPS, THETA).with_norm_weight_dtype(DTYPE_BF16)
+    page_config = kpw.Config(hkv, d, g.page_bytes, kv_dtype=DTYPE_FP8_E4M3FN if fp8_pages else DTYPE_BF16)
+    page_shape = kpw.Shape(total, kpw.PageTableLayout(w.num_req_slots, g.num_gqa_layers, g.num_blocks, g.num_page_ids_per_block))
+    config = gpu_runner.component_config(w, sliced_q.Config)
+    variant = sdpa.ExecutionVariant.sliced_q(config.sdpa_config(), sdpa.MAP_Q_TOKENS_AND_HEADS, tile, 64, hq // hkv)
+    ranges, templates, _ = helpers.fixed_slice_plan(histories, q_lens, tile, 1 << 30)
+    ranges = np.asarray(ranges, dtype=np.uint32).reshape(-1, 2)
+    templates = np.asarray(templates, dtype=np.uint32).reshape(-1, 3)
+    compute = sliced_q.Compute(config, variant, sliced_q.Shape(total, ranges.shape[0], templates.shape[0]), direct=True)
+    visible_d, ranges_d, templates_d = to(w.visible), to(ranges), to(templates)
+    weight_q_d, weight_k_d, projection_d = to(weight_q), to(weight_k), to(projection)
+    torch.cuda.synchronize()
+
+    print(f"projection to gated output: Hq{hq}/Hkv{hkv}/D{d} tile {tile} fp8_pages={fp8_pages}", flush=True)
+    active = ReplayU32.fixed(total)
+    qgkv_split.Compute(qgkv_split.Config.bf16(hq, hkv, d)).invoke(qgkv_split.Shape(total), qgkv=projection_d, q=q_split, g=g_split, k=k_split,
+                                                                    v=v_split, num_active_tokens=active)
+    rnr.Compute(norm_q).invoke(rnr.Shape(total), input=q_split, norm_weight=weight_q_d, flat_token_indices=positions_d, output=q_rows,
+                               num_active_tokens=active)
+    fused_writer.Compute(norm_k, page_config).invoke(page_shape, pages=pages, k=k_split, v=v_split, norm_weight=weight_k_d, req_slots=slots_d,
+                                                     flat_token_indices=positions_d, page_ids=table_d, num_active_tokens=active,
+                                                     page_table_index=ReplayU32.fixed(w.layer))
+    compute.invoke_direct(q=q_rows, kv_pages=pages, req_slots=slots_d, page_ids=table_d, visible_kv_token_ranges=visible_d,
+                          q_token_ranges=ranges_d, sdpa_map_task_templates=templates_d, output=out, page_table_index=ReplayU32.fixed(w.layer),
+                          num_active_tokens=active, num_active_q_token_tiles=ReplayU32.fixed(ranges.shape[0]), gates=g_split)
+    torch.cuda.synchronize()
+
+    host = lambda t: t.cpu().numpy().view(np.uint16)  # noqa: E731
+    assert np.array_equal(host(q_split), q_raw) and np.array_equal(host(g_split), gate_bits)
+    assert np.array_equal(host(k_split), k_raw) and np.array_equal(host(v_split), v_new)
+
+    def gated(attention_f32):   # the gate sees the bf16-rounded attention output (gqa_activation_gate.metal:19-39)
+        return oracle.bf16_bits_to_f32(oracle.gate_bf16(oracle.f32_to_bf16_bits(attention_f32).reshape(-1), gate_bits.reshape(-1)))
+
+    actual = gpu_runner.bf16_tensor_to_f32(out)
+    # the oracle on exactly the Q rows and page bytes the producers left in memory
+    pages_device = pages.cpu().numpy().view(np.uint8).reshape(w.kv_pages.shape)
+    from_device = helpers.expected_output(dataclasses.replace(w, q_bits=host(q_rows), kv_pages=pages_device))
+    helpers.assert_parity(actual, gated(from_device), "gated attention over the rows the producers just wrote", abs_tol=4e-3)
+    # and the oracle's own chain from the projection rows
+    q_expected = oracle.rms_norm_rope(q_raw, weight_q, positions, hq, d, d, EPS, THETA, io_bf16=True, weight_bf16=True)
+    k_expected = oracle.rms_norm_rope(k_raw, weight_k, positions, hkv, d, d, EPS, THETA, io_bf16=True, weight_bf16=True)
+    pages_expected = oracle.kv_page_write(w.kv_pages.reshape(-1), k_expected, v_new, w.req_slots, positions, w.page_ids, total, w.layer,
+                                          g.num_gqa_layers, g.num_blocks, g.num_page_ids_per_block, hkv, d, tpp, g.page_bytes, fp8_pages)
+    chain = helpers.expected_output(dataclasses.replace(w, q_bits=q_expected, kv_pages=pages_expected.reshape(w.kv_pages.shape)))
+    helpers.assert_parity(actual, gated(chain), "projection rows to gated output on one stream", abs_tol=6e-3)
