@@ -530,6 +530,34 @@ int khm_k_norm_rope_page_write(const khm_rms_norm_rope_config* norm_config, cons
                                khm_replay_u32 num_active_tokens, khm_replay_u32 page_table_index,
                                const uint32_t* replay_parameters, void* stream);
 
+/* The projection split, Q RMSNorm + RoPE, K RMSNorm + RoPE and the K/V page write as one launch: everything GQA::record
+ * enqueues between the input projection and the SDPA (crates/inference-executor-metal/src/attn/gqa/backend.rs:358-412;
+ * qgkv_split.rs:187-236, rms_norm_rope.rs:286-403, kv_page_write.rs:136-262), reading the projection rows once and
+ * writing only what the SDPA and the gate read.  q_output, gate_output and the pages receive exactly the bytes that
+ * khm_gqa_qgkv_split (gated != 0; khm_gqa_qkv_split otherwise, gate_output unused), khm_rms_norm_rope on the Q rows and
+ * khm_k_norm_rope_page_write on the K and V rows would have left there.  q_norm_config.num_heads is Hq,
+ * k_norm_config.num_heads is Hkv = page_config.num_kv_heads; both configs must agree in head_dim, rope_dim, rope_theta,
+ * rope_scaling and norm_weight_dtype (eps may differ) and take BF16 rows.  shape.num_total_token_writes is the token
+ * count of all three steps.  KHM_ERR_UNSUPPORTED outside the vector path (head_dim > 512, head_dim or rope_dim / 2 no
+ * multiple of 8, buffers not 16-byte aligned): the separate calls cover those. */
+typedef struct khm_gqa_projection_norm_rope_page_write_buffers {
+    khm_buffer projection;    /* bf16 [T][(2 or 1) * Hq * D + 2 * Hkv * D], read only */
+    khm_buffer q_norm_weight; /* [D] */
+    khm_buffer k_norm_weight; /* [D] */
+    khm_buffer q_output;      /* bf16 [T][Hq][D]: normalised, rotated Q rows */
+    khm_buffer gate_output;   /* bf16 [T][Hq][D]: gate rows as they are (gated form) */
+    khm_buffer pages;
+    khm_buffer req_slots;
+    khm_buffer flat_token_indices;
+    khm_buffer page_ids;
+} khm_gqa_projection_norm_rope_page_write_buffers;
+int khm_gqa_projection_norm_rope_page_write(uint32_t gated, const khm_rms_norm_rope_config* q_norm_config,
+                                            const khm_rms_norm_rope_config* k_norm_config,
+                                            const khm_kv_page_write_config* page_config, const khm_kv_page_write_shape* shape,
+                                            const khm_gqa_projection_norm_rope_page_write_buffers* buffers,
+                                            khm_replay_u32 num_active_tokens, khm_replay_u32 page_table_index,
+                                            const uint32_t* replay_parameters, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Executor-side host logic that feeds the component (CPU only, no HIP calls)
  * ------------------------------------------------------------------------------------------ */

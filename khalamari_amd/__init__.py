@@ -7,4 +7,4 @@ host logic live in `lib/libkhm_gqa_sdpa.so` (sources under `csrc/`, ABI in `incl
 """
 from . import _lib  # noqa: F401
 
-__all__ = ["_lib", "sdpa", "sliced_kv", "sliced_q", "activation_gate", "qgkv_split", "qkv_split", "kv_page_write", "bidi_block_sdpa", "bidi_block_metadata", "rms_norm_rope", "selector", "batch_metadata", "replay"]
+__all__ = ["_lib", "sdpa", "sliced_kv", "sliced_q", "activation_gate", "qgkv_split", "qkv_split", "kv_page_write", "bidi_block_sdpa", "bidi_block_metadata", "rms_norm_rope", "k_norm_rope_page_write", "projection_norm_rope_page_write", "selector", "batch_metadata", "replay"]

@@ -240,6 +240,11 @@ class KNormRopePageWriteBuffers(ctypes.Structure):
                 ("flat_token_indices", Buffer), ("page_ids", Buffer)]
 
 
+class ProjectionNormRopePageWriteBuffers(ctypes.Structure):
+    _fields_ = [("projection", Buffer), ("q_norm_weight", Buffer), ("k_norm_weight", Buffer), ("q_output", Buffer),
+                ("gate_output", Buffer), ("pages", Buffer), ("req_slots", Buffer), ("flat_token_indices", Buffer), ("page_ids", Buffer)]
+
+
 # Every symbol `include/khm_gqa_sdpa.h` declares; checked by tests/test_abi.py.
 EXPORTED_SYMBOLS = (
     "khm_last_error", "khm_version",
@@ -262,7 +267,7 @@ EXPORTED_SYMBOLS = (
     "khm_bidi_block_sdpa",
     "khm_bidi_block_capacity_new", "khm_bidi_block_select", "khm_bidi_block_metadata_compute",
     "khm_rms_norm_rope_yarn_correction_range", "khm_rms_norm_rope_kernel_parameters", "khm_rms_norm_rope",
-    "khm_k_norm_rope_page_write",
+    "khm_k_norm_rope_page_write", "khm_gqa_projection_norm_rope_page_write",
     "khm_replay_bucket_policy_create", "khm_replay_bucket_policy_destroy", "khm_replay_bucket_policy_max_capacity",
     "khm_replay_bucket_policy_buckets", "khm_replay_bucket_policy_capacity", "khm_replay_bucket_policy_capacity_allow_zero",
     "khm_request_shapes_from_batch",
@@ -373,6 +378,10 @@ def lib() -> ctypes.CDLL:
     handle.khm_k_norm_rope_page_write.argtypes = [ctypes.POINTER(RmsNormRopeConfig), ctypes.POINTER(KvPageWriteConfig),
                                                   ctypes.POINTER(KvPageWriteShape), ctypes.POINTER(KNormRopePageWriteBuffers), ReplayU32,
                                                   ReplayU32, ctypes.c_void_p, ctypes.c_void_p]
+    handle.khm_gqa_projection_norm_rope_page_write.argtypes = [u32, ctypes.POINTER(RmsNormRopeConfig), ctypes.POINTER(RmsNormRopeConfig),
+                                                               ctypes.POINTER(KvPageWriteConfig), ctypes.POINTER(KvPageWriteShape),
+                                                               ctypes.POINTER(ProjectionNormRopePageWriteBuffers), ReplayU32, ReplayU32,
+                                                               ctypes.c_void_p, ctypes.c_void_p]
     _lib = handle
     return handle
 

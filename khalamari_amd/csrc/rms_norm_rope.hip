@@ -36,6 +36,9 @@ struct RmsNormRopeParams {
     float attention_factor;
     uint32_t tokens_per_block;      // rows kernels: tokens a block serves (more than one when there are few heads)
     uint32_t row_slots_per_token_shift;  // rows kernels: log2 of the row slots of a block that one token takes
+    uint32_t input_row_stride;      // rows kernels: elements from a token's first input row to the next token's (H * D when packed)
+    uint32_t input_head_stride;     // rows kernels: elements from a head's input row to the next head's (D when packed)
+    void* gate_output;              // projection rows kernel: [T][H][D] rows copied from the D elements behind each input row
     float inverse_frequencies[kMaxRopeHalf];
 };
 
@@ -190,9 +193,33 @@ constexpr int kMaxTokensPerBlock = 16;
 // PAGES: 0 writes the rows to p.output; 1 / 2 scatter them, as K rows, straight into bf16 / FP8 E4M3FN pages through
 // the page table and copy the V rows of the same (token, KV head) beside them: RMSNorm + RoPE of K and the K/V page write
 // in one pass, the bf16 value the two-kernel sequence would have stored in between being the one that is encoded.
-template <typename T, typename W, uint32_t LPR, uint32_t PARTNER, int PAGES>
-__device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, const PageWriteParams* pages) {
+// What differs between the row sets one launch can serve (Q rows to an output buffer, K rows to pages); the rotation
+// table, positions and active count are shared (RmsNormRopeParams).
+struct RowsRole {
+    const void* input;           // first element of token 0, head 0
+    const void* norm_weight;     // [D]
+    void* output;                // PAGES == 0: [T][H][D]
+    void* gate_output;           // GATE: [T][H][D]
+    uint32_t num_heads;
+    uint32_t input_row_stride;   // elements
+    uint32_t input_head_stride;  // elements
+    uint32_t v_row_stride;       // PAGES != 0: elements from a token's V rows to the next token's (heads are D apart)
+    float eps;
+    uint32_t tokens_per_block;
+    uint32_t row_slots_per_token_shift;
+};
+__device__ __forceinline__ RowsRole role_of(const RmsNormRopeParams& p) {
+    return RowsRole{p.input, p.norm_weight, p.output, p.gate_output, p.num_heads, p.input_row_stride, p.input_head_stride,
+                    p.num_heads * p.head_dim, p.eps, p.tokens_per_block, p.row_slots_per_token_shift};
+}
+
+// GATE: the D elements behind every input row (the gate half of a gated projection's head pair) are copied to
+// role.gate_output as they are.  `sines` / `cosines` are the block's LDS tables, [kMaxTokensPerBlock * kMaxRopeHalf] each.
+template <typename T, typename W, uint32_t LPR, uint32_t PARTNER, int PAGES, bool GATE>
+__device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, const RowsRole& role, const PageWriteParams* pages,
+                                                   uint32_t block_x, uint32_t block_y, float* sines, float* cosines) {
     static_assert(PAGES == 0 || sizeof(T) == 2, "pages are written from bf16 rows");
+    static_assert(!GATE || (PAGES == 0 && sizeof(T) == 2), "gate rows are copied beside bf16 output rows");
     constexpr uint32_t kRowsPerWave = 64u / LPR;
     constexpr int kRows = PAGES != 0 ? kPageRowsInFlight : kRowsInFlight;   // row groups of a wave
     constexpr uint32_t kRowSlots = 4 * kRows * kRowsPerWave;   // (token, head) rows a block holds
@@ -201,9 +228,9 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
     // Row slot s of the block belongs to token s >> shift of the block's tokens and to head s & (2^shift - 1) of this
     // block's head group: one token per block when the heads fill the slots, several when there are few heads (the K
     // rows of a grouped-query model), so that every wave has rows and a token's sines and cosines are shared by its heads.
-    const uint32_t tokens_per_block = p.tokens_per_block, slot_shift = p.row_slots_per_token_shift;
+    const uint32_t tokens_per_block = role.tokens_per_block, slot_shift = role.row_slots_per_token_shift;
     const uint32_t num_active_tokens = resolve_u32(p.num_active_tokens, p.replay_parameters);
-    const uint32_t first_token = blockIdx.x * tokens_per_block;
+    const uint32_t first_token = block_x * tokens_per_block;
     if (first_token >= num_active_tokens) return;
     const uint32_t sub_row = lane / LPR;
     const uint32_t first = (lane % LPR) * 8;
@@ -213,6 +240,7 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
     const int partner_lane = ((int)lane + (lower ? (int)(rope_half / 8) : -(int)(rope_half / 8))) & 63;
 
     typename Row8<T>::Raw raw[kRows];   // rows stay as loaded until their turn: half the registers of eight floats
+    typename Row8<T>::Raw gate_raw[GATE ? kRows : 1];
     uint32_t heads[kRows], tokens[kRows], local_tokens[kRows];
     bool valid[kRows];
 #pragma unroll
@@ -220,10 +248,14 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
         const uint32_t slot = (j * 4 + wave) * kRowsPerWave + sub_row;
         local_tokens[j] = slot >> slot_shift;
         tokens[j] = first_token + local_tokens[j];
-        heads[j] = blockIdx.y * kRowSlots + (slot & ((1u << slot_shift) - 1u));
-        valid[j] = holds && heads[j] < p.num_heads && local_tokens[j] < tokens_per_block && tokens[j] < num_active_tokens;
+        heads[j] = block_y * kRowSlots + (slot & ((1u << slot_shift) - 1u));
+        valid[j] = holds && heads[j] < role.num_heads && local_tokens[j] < tokens_per_block && tokens[j] < num_active_tokens;
         raw[j] = Row8<T>::zero();
-        if (valid[j]) raw[j] = Row8<T>::load_raw(static_cast<const T*>(p.input) + ((uint64_t)tokens[j] * p.num_heads + heads[j]) * p.head_dim + first);
+        const T* source = static_cast<const T*>(role.input) + (uint64_t)tokens[j] * role.input_row_stride + (uint64_t)heads[j] * role.input_head_stride + first;
+        if (valid[j]) raw[j] = Row8<T>::load_raw(source);
+        if constexpr (GATE) {
+            if (valid[j]) gate_raw[j] = Row8<T>::load_raw(source + p.head_dim);
+        }
     }
     // Page writes: the V chunks and the page-table walk (request slot, position -> page id) of every row are requested
     // here, beside the K rows, so that their round trips pass under the sine/cosine evaluation and the block barrier
@@ -238,15 +270,13 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
             v_chunk[j] = make_uint4(0, 0, 0, 0);
             target[j] = PageTarget{0, 0};
             if (valid[j]) {
-                v_chunk[j] = *reinterpret_cast<const uint4*>(pages->flat_v + ((uint64_t)tokens[j] * p.num_heads + heads[j]) * p.head_dim + first);
+                v_chunk[j] = *reinterpret_cast<const uint4*>(pages->flat_v + (uint64_t)tokens[j] * role.v_row_stride + heads[j] * p.head_dim + first);
                 target[j] = page_target_of(*pages, pages->req_slots[tokens[j]], pages->flat_token_indices[tokens[j]], layer, heads[j], first,
                                            kElementBytes);
             }
         }
     }
     // the rotation tables of the block's tokens, one sine/cosine evaluation per token and rotary pair
-    __shared__ __align__(16) float sines[kMaxTokensPerBlock * kMaxRopeHalf];
-    __shared__ __align__(16) float cosines[kMaxTokensPerBlock * kMaxRopeHalf];
     for (uint32_t entry = threadIdx.x; entry < tokens_per_block * rope_half; entry += 256) {
         const uint32_t local = entry / rope_half, pair = entry - local * rope_half;
         if (first_token + local < num_active_tokens) {
@@ -255,8 +285,14 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
         }
     }
     typename Row8<W>::Raw w_raw = Row8<W>::zero();
-    if (holds) w_raw = Row8<W>::load_raw(static_cast<const W*>(p.norm_weight) + first);
+    if (holds) w_raw = Row8<W>::load_raw(static_cast<const W*>(role.norm_weight) + first);
     __syncthreads();
+    if constexpr (GATE) {   // the gate rows have arrived with the input rows: pass them on before the arithmetic
+#pragma unroll
+        for (int j = 0; j < kRows; ++j) {
+            if (valid[j]) store_streaming(static_cast<T*>(role.gate_output) + ((uint64_t)tokens[j] * role.num_heads + heads[j]) * p.head_dim + first, gate_raw[j]);
+        }
+    }
     const float inverse_dim = 1.0f / (float)p.head_dim;
     float sine[8], cosine[8];
 #pragma unroll
@@ -271,7 +307,7 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
         for (int i = 0; i < 8; ++i) acc += x[i] * x[i];
         acc = sum_in_row<LPR>(acc, lane);
         // v_rsq_f32 (1 ulp) and one Newton step, which leaves the error below that of a correctly rounded rsqrt's input
-        const float mean = acc * inverse_dim + p.eps;
+        const float mean = acc * inverse_dim + role.eps;
         float inv_rms = __builtin_amdgcn_rsqf(mean);
         inv_rms = inv_rms * __builtin_fmaf(-0.5f * mean * inv_rms, inv_rms, 1.5f);
         if (rotated && valid[j] && (j == 0 || tokens_per_block > 1)) {   // one token per block: every row shares the first load
@@ -301,7 +337,7 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
         }
         if (!valid[j]) continue;
         if constexpr (PAGES == 0) {
-            Row8<T>::store(static_cast<T*>(p.output) + ((uint64_t)tokens[j] * p.num_heads + heads[j]) * p.head_dim + first, out);
+            Row8<T>::store(static_cast<T*>(role.output) + ((uint64_t)tokens[j] * role.num_heads + heads[j]) * p.head_dim + first, out);
         } else {
             const uint4 k_chunk = make_uint4(pack_bf16x2(out[0], out[1]), pack_bf16x2(out[2], out[3]), pack_bf16x2(out[4], out[5]), pack_bf16x2(out[6], out[7]));
             uint8_t* k_target = pages->pages + target[j].k_offset;
@@ -317,14 +353,44 @@ __device__ __forceinline__ void rms_norm_rope_rows(const RmsNormRopeParams& p, c
     }
 }
 
+#define KHM_ROTATION_TABLES                                                          \
+    __shared__ __align__(16) float sines[kMaxTokensPerBlock * kMaxRopeHalf];         \
+    __shared__ __align__(16) float cosines[kMaxTokensPerBlock * kMaxRopeHalf]
+
 template <typename T, typename W, uint32_t LPR, uint32_t PARTNER>
 __global__ __launch_bounds__(256) void rms_norm_rope_rows_kernel(const RmsNormRopeParams p) {
-    rms_norm_rope_rows<T, W, LPR, PARTNER, 0>(p, nullptr);
+    KHM_ROTATION_TABLES;
+    rms_norm_rope_rows<T, W, LPR, PARTNER, 0, false>(p, role_of(p), nullptr, blockIdx.x, blockIdx.y, sines, cosines);
 }
 
 template <typename W, uint32_t LPR, uint32_t PARTNER, bool FP8_PAGES>
 __global__ __launch_bounds__(256) void k_norm_rope_page_write_kernel(const RmsNormRopeParams p, const PageWriteParams pages) {
-    rms_norm_rope_rows<uint16_t, W, LPR, PARTNER, FP8_PAGES ? 2 : 1>(p, &pages);
+    KHM_ROTATION_TABLES;
+    rms_norm_rope_rows<uint16_t, W, LPR, PARTNER, FP8_PAGES ? 2 : 1, false>(p, role_of(p), &pages, blockIdx.x, blockIdx.y, sines, cosines);
+}
+
+// Everything between the input projection and the SDPA in one launch (the reference records qgkv_split, q_norm_rope,
+// k_norm_rope and kv_page_write: crates/inference-executor-metal/src/attn/gqa/backend.rs:358-412).  The first
+// q_blocks blocks take the Q rows straight from the projection rows (head pairs [q | gate] when GATED, gate halves copied
+// to their own buffer on the way), the others the K rows and, beside them, the V rows into the pages.  `p` describes the
+// Q rows; the K rows differ in what `k_role` holds.
+struct ProjectionBlocks {
+    uint32_t q_blocks;     // blocks of the Q role, laid out [head group][token group]
+    uint32_t q_blocks_x;   // token groups of the Q role
+    uint32_t k_blocks_x;   // token groups of the K role
+};
+template <typename W, uint32_t LPR, uint32_t PARTNER, bool FP8_PAGES, bool GATED>
+__global__ __launch_bounds__(256) void projection_norm_rope_page_write_kernel(const RmsNormRopeParams p, const RowsRole k_role,
+                                                                              const PageWriteParams pages, const ProjectionBlocks blocks) {
+    KHM_ROTATION_TABLES;
+    if (blockIdx.x < blocks.q_blocks) {
+        const uint32_t block_y = blockIdx.x / blocks.q_blocks_x;
+        rms_norm_rope_rows<uint16_t, W, LPR, PARTNER, 0, GATED>(p, role_of(p), nullptr, blockIdx.x - block_y * blocks.q_blocks_x, block_y, sines, cosines);
+    } else {
+        const uint32_t index = blockIdx.x - blocks.q_blocks;
+        const uint32_t block_y = index / blocks.k_blocks_x;
+        rms_norm_rope_rows<uint16_t, W, LPR, PARTNER, FP8_PAGES ? 2 : 1, false>(p, k_role, &pages, index - block_y * blocks.k_blocks_x, block_y, sines, cosines);
+    }
 }
 
 // RopeScaling::yarn_kernel_parameters (rms_norm_rope.rs:206-243).
@@ -462,6 +528,9 @@ static int fill_rms_norm_rope_params(const khm_rms_norm_rope_config* config, uin
     p.head_dim = config->head_dim;
     p.rope_dim = config->rope_dim;
     p.eps = config->eps;
+    p.input_row_stride = config->num_heads * config->head_dim;
+    p.input_head_stride = config->head_dim;
+    p.gate_output = nullptr;
     *out = p;
     return KHM_OK;
 }
@@ -584,5 +653,112 @@ extern "C" int khm_k_norm_rope_page_write(const khm_rms_norm_rope_config* norm_c
     else launch(float{}, std::false_type{});
     const hipError_t status = hipGetLastError();
     if (status != hipSuccess) return fail(KHM_ERR_HIP, "K RMSNorm/RoPE page write launch failed: %s", hipGetErrorString(status));
+    return KHM_OK;
+}
+
+static bool same_rotation(const khm_rms_norm_rope_config& a, const khm_rms_norm_rope_config& b) {
+    const khm_rope_scaling &x = a.rope_scaling, &y = b.rope_scaling;
+    return a.head_dim == b.head_dim && a.rope_dim == b.rope_dim && a.rope_theta == b.rope_theta && x.kind == y.kind &&
+           (x.kind != KHM_ROPE_SCALING_YARN ||
+            (x.factor == y.factor && x.attention_factor == y.attention_factor && x.beta_fast == y.beta_fast && x.beta_slow == y.beta_slow &&
+             x.original_max_position_embeddings == y.original_max_position_embeddings && x.truncate == y.truncate));
+}
+
+// The projection split, Q RMSNorm + RoPE, K RMSNorm + RoPE and the K/V page write in one launch: what GQA::record enqueues
+// between the input projection and the SDPA (crates/inference-executor-metal/src/attn/gqa/backend.rs:358-412), with no
+// q, k, v or normalised-K rows in memory in between.  Outputs are exactly what khm_gqa_qgkv_split (or khm_gqa_qkv_split),
+// khm_rms_norm_rope on the Q rows and khm_k_norm_rope_page_write leave in q_output, gate_output and the pages.
+extern "C" int khm_gqa_projection_norm_rope_page_write(uint32_t gated, const khm_rms_norm_rope_config* q_norm_config,
+                                                       const khm_rms_norm_rope_config* k_norm_config,
+                                                       const khm_kv_page_write_config* page_config, const khm_kv_page_write_shape* shape,
+                                                       const khm_gqa_projection_norm_rope_page_write_buffers* buffers,
+                                                       khm_replay_u32 num_active_tokens, khm_replay_u32 page_table_index,
+                                                       const uint32_t* replay_parameters, void* stream) {
+    clear_error();
+    KHM_REQUIRE(q_norm_config != nullptr && k_norm_config != nullptr && page_config != nullptr && shape != nullptr && buffers != nullptr,
+                "configs, shape and buffers must not be null");
+    if (int status = validate_rms_norm_rope_config(q_norm_config)) return status;
+    if (int status = validate_rms_norm_rope_config(k_norm_config)) return status;
+    KHM_REQUIRE(k_norm_config->num_heads == page_config->num_kv_heads && k_norm_config->head_dim == page_config->head_dim,
+                "K RMSNorm/RoPE rows [%u][%u] do not match the page writer's KV heads [%u][%u]", k_norm_config->num_heads,
+                k_norm_config->head_dim, page_config->num_kv_heads, page_config->head_dim);
+    KHM_REQUIRE(q_norm_config->dtype == KHM_DTYPE_BF16 && k_norm_config->dtype == KHM_DTYPE_BF16,
+                "the fused projection RMSNorm/RoPE page write takes BF16 projection rows");
+    KHM_REQUIRE(same_rotation(*q_norm_config, *k_norm_config) && q_norm_config->norm_weight_dtype == k_norm_config->norm_weight_dtype,
+                "the fused projection RMSNorm/RoPE page write needs the same head_dim, rotation and weight dtype for Q and K");
+    const uint32_t tokens = shape->num_total_token_writes;
+    const uint32_t head_dim = q_norm_config->head_dim, hq = q_norm_config->num_heads, hkv = k_norm_config->num_heads;
+    const uint64_t q_heads_in_row = (gated ? 2ull : 1ull) * hq;
+    const uint64_t row_heads = q_heads_in_row + 2ull * hkv;
+    const __uint128_t elements = (__uint128_t)tokens * row_heads * head_dim;
+    KHM_REQUIRE(tokens > 0 && elements <= 0xffffffffull, "%s elements exceeds the shader u32 count domain",
+                gated ? "GQA projection" : "ungated GQA projection");
+    const uint64_t width = row_heads * head_dim;
+    const uint64_t q_bytes = (uint64_t)tokens * hq * head_dim * 2;
+    KHM_REQUIRE(buffers->projection.ptr != nullptr && buffers->projection.len_bytes >= (uint64_t)elements * 2,
+                "projection buffer holds %llu bytes, needs %llu", (unsigned long long)buffers->projection.len_bytes,
+                (unsigned long long)((uint64_t)elements * 2));
+    if (gated)
+        KHM_REQUIRE(buffers->gate_output.ptr != nullptr && buffers->gate_output.len_bytes >= q_bytes, "gate_output buffer holds %llu bytes, needs %llu",
+                    (unsigned long long)buffers->gate_output.len_bytes, (unsigned long long)q_bytes);
+    // K and V rows as windows of the projection rows
+    const uint64_t k_offset = q_heads_in_row * head_dim * 2, v_offset = k_offset + (uint64_t)hkv * head_dim * 2;
+    uint8_t* base = static_cast<uint8_t*>(buffers->projection.ptr);
+    const khm_buffer k_window{base + k_offset, buffers->projection.len_bytes - k_offset};
+    const khm_buffer v_window{base + v_offset, buffers->projection.len_bytes - v_offset};
+    const khm_kv_page_write_buffers page_buffers{buffers->pages, k_window, v_window, buffers->req_slots, buffers->flat_token_indices, buffers->page_ids};
+    PageWriteParams pages{};
+    if (int status = fill_page_write_params(page_config, shape, &page_buffers, num_active_tokens, page_table_index, replay_parameters, &pages))
+        return status;
+    RmsNormRopeParams p{}, k_params{};
+    if (int status = fill_rms_norm_rope_params(q_norm_config, tokens, buffers->projection, buffers->q_norm_weight, buffers->flat_token_indices,
+                                               &buffers->q_output, num_active_tokens, replay_parameters, &p))
+        return status;
+    if (int status = fill_rms_norm_rope_params(k_norm_config, tokens, k_window, buffers->k_norm_weight, buffers->flat_token_indices, nullptr,
+                                               num_active_tokens, replay_parameters, &k_params))
+        return status;
+    const uintptr_t address_bits = (uintptr_t)base | (uintptr_t)p.output | (uintptr_t)p.norm_weight | (uintptr_t)k_params.norm_weight |
+                                   (uintptr_t)pages.pages | (uintptr_t)buffers->gate_output.ptr | (uintptr_t)(width * 2);
+    const RowsGeometry q_geometry = rows_geometry(*q_norm_config, tokens, address_bits);
+    const RowsGeometry k_geometry = rows_geometry(*k_norm_config, tokens, address_bits, kPageRowsInFlight);
+    if (!q_geometry.fits || !k_geometry.fits || page_config->page_bytes % 16 != 0)
+        return fail(KHM_ERR_UNSUPPORTED, "the fused projection RMSNorm/RoPE page write needs 16-byte aligned buffers and rows, head_dim <= 512, and "
+                                         "head_dim and rope_dim / 2 multiples of 8: run the split, khm_rms_norm_rope and khm_kv_page_write instead");
+    p.tokens_per_block = q_geometry.tokens_per_block;
+    p.row_slots_per_token_shift = q_geometry.slot_shift;
+    p.input_row_stride = (uint32_t)width;
+    p.input_head_stride = gated ? 2 * head_dim : head_dim;
+    p.gate_output = gated ? buffers->gate_output.ptr : nullptr;
+    const RowsRole k_role{k_params.input, k_params.norm_weight, nullptr, nullptr, hkv, (uint32_t)width, head_dim, (uint32_t)width, k_norm_config->eps,
+                          k_geometry.tokens_per_block, k_geometry.slot_shift};
+    const uint64_t q_blocks = (uint64_t)q_geometry.grid.x * q_geometry.grid.y, k_blocks = (uint64_t)k_geometry.grid.x * k_geometry.grid.y;
+    KHM_REQUIRE(q_blocks + k_blocks <= 0x7fffffffull, "the fused projection RMSNorm/RoPE page write needs %llu blocks, more than one launch covers",
+                (unsigned long long)(q_blocks + k_blocks));
+    const ProjectionBlocks blocks{(uint32_t)q_blocks, q_geometry.grid.x, k_geometry.grid.x};
+    const dim3 grid((uint32_t)(q_blocks + k_blocks));
+    hipStream_t hip_stream = static_cast<hipStream_t>(stream);
+    const bool weight_bf16 = q_norm_config->norm_weight_dtype == KHM_DTYPE_BF16, fp8_pages = page_config->kv_dtype == KHM_DTYPE_FP8_E4M3FN;
+    auto launch = [&](auto weight_tag, auto fp8_tag, auto gated_tag) {
+        typedef decltype(weight_tag) W;
+        constexpr bool FP8 = decltype(fp8_tag)::value, GATED = decltype(gated_tag)::value;
+#define KHM_ROWS_CASE(LPR, PARTNER)                                                                                                          \
+    if (q_geometry.lanes_per_row == LPR && q_geometry.partner == PARTNER) {                                                                  \
+        hipLaunchKernelGGL((projection_norm_rope_page_write_kernel<W, LPR, PARTNER, FP8, GATED>), grid, dim3(256), 0, hip_stream, p, k_role, \
+                           pages, blocks);                                                                                                   \
+        return;                                                                                                                              \
+    }
+        KHM_ROWS_CASES(KHM_ROWS_CASE)
+#undef KHM_ROWS_CASE
+    };
+    auto with_gate = [&](auto weight_tag, auto fp8_tag) {
+        if (gated) launch(weight_tag, fp8_tag, std::true_type{});
+        else launch(weight_tag, fp8_tag, std::false_type{});
+    };
+    if (weight_bf16 && fp8_pages) with_gate(uint16_t{}, std::true_type{});
+    else if (weight_bf16) with_gate(uint16_t{}, std::false_type{});
+    else if (fp8_pages) with_gate(float{}, std::true_type{});
+    else with_gate(float{}, std::false_type{});
+    const hipError_t status = hipGetLastError();
+    if (status != hipSuccess) return fail(KHM_ERR_HIP, "projection RMSNorm/RoPE page write launch failed: %s", hipGetErrorString(status));
     return KHM_OK;
 }
