@@ -511,7 +511,6 @@ def producer_rows(device, steps: int = 20) -> dict:
     nbytes = 2 * split_config.projection_bytes(split_shape)
     result["qgkv_split"] = {"workload": f"projection rows {tokens}x(2x{hq}+2x{hkv})x{d} bf16 -> q, g, k, v", "kernel_us": us,
                             "algorithmic_bytes": nbytes, "gbps": nbytes / us / 1e3, "roofline_frac": nbytes / us / 1e3 / HBM_PEAK_GBPS}
-    del projection, split_q, split_g, split_k, split_v
 
     q = torch.randn((tokens, hq, d), device=device, dtype=torch.float32, generator=generator).to(torch.bfloat16)
     q_out = torch.empty_like(q)
@@ -559,6 +558,31 @@ def producer_rows(device, steps: int = 20) -> dict:
     result["k_norm_rope_page_write"] = {"workload": f"K RMSNorm + RoPE and K/V rows {tokens}x{hkv}x{d} bf16 -> FP8 E4M3FN pages, one launch",
                                         "kernel_us": us, "algorithmic_bytes": nbytes, "gbps": nbytes / us / 1e3,
                                         "roofline_frac": nbytes / us / 1e3 / HBM_PEAK_GBPS, "two_launches_us": separate_us}
+
+    # everything between the input projection and the SDPA in one launch, beside the three launches it replaces
+    # (projection split, Q norm/rope, fused K writer)
+    from khalamari_amd import projection_norm_rope_page_write
+
+    q_config, k_config = rms_norm_rope.Config.bf16(hq, d, d, 1e-6, 1_000_000.0), rms_norm_rope.Config.bf16(hkv, d, d, 1e-6, 1_000_000.0)
+    prologue = projection_norm_rope_page_write.Compute(q_config, k_config, kv_page_write.Config(hkv, d, page_bytes))
+    q_norm = rms_norm_rope.Compute(q_config)
+
+    def three_launches():
+        split.invoke(split_shape, qgkv=projection, q=split_q, g=split_g, k=split_k, v=split_v, num_active_tokens=ReplayU32.fixed(tokens))
+        q_norm.invoke(rms_norm_rope.Shape(tokens), input=split_q, norm_weight=weight, flat_token_indices=positions, output=q_out,
+                      num_active_tokens=ReplayU32.fixed(tokens))
+        fused.invoke(shape, pages=pages, k=split_k, v=split_v, norm_weight=weight, req_slots=req_slots, flat_token_indices=positions,
+                     page_ids=page_ids, num_active_tokens=ReplayU32.fixed(tokens), page_table_index=ReplayU32.fixed(0))
+
+    separate_us = timed(three_launches)
+    us = timed(lambda: prologue.invoke(shape, projection=projection, q_norm_weight=weight, k_norm_weight=weight, q_output=q_out,
+                                       gate_output=split_g, pages=pages, req_slots=req_slots, flat_token_indices=positions, page_ids=page_ids,
+                                       num_active_tokens=ReplayU32.fixed(tokens), page_table_index=ReplayU32.fixed(0)))
+    nbytes = split_config.projection_bytes(split_shape) + 2 * q.numel() * 2 + 2 * flat_k.numel()
+    result["projection_norm_rope_page_write"] = {
+        "workload": f"projection rows {tokens}x(2x{hq}+2x{hkv})x{d} bf16 -> Q rows (norm + RoPE), gate rows, K (norm + RoPE) / V into FP8 E4M3FN "
+                    "pages, one launch", "kernel_us": us, "algorithmic_bytes": nbytes, "gbps": nbytes / us / 1e3,
+        "roofline_frac": nbytes / us / 1e3 / HBM_PEAK_GBPS, "three_launches_us": separate_us}
     return result
 
 

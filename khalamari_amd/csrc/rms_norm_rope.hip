@@ -734,6 +734,8 @@ extern "C" int khm_gqa_projection_norm_rope_page_write(uint32_t gated, const khm
     const uint64_t q_blocks = (uint64_t)q_geometry.grid.x * q_geometry.grid.y, k_blocks = (uint64_t)k_geometry.grid.x * k_geometry.grid.y;
     KHM_REQUIRE(q_blocks + k_blocks <= 0x7fffffffull, "the fused projection RMSNorm/RoPE page write needs %llu blocks, more than one launch covers",
                 (unsigned long long)(q_blocks + k_blocks));
+    // (Running the blocks in token order instead, the Q blocks of four tokens and then their K block, changes nothing:
+    // 212.6 against 213.5 us on 16384 tokens; two or one row group in flight in the Q blocks: 218.5 / 217.1 against 214.2 us.)
     const ProjectionBlocks blocks{(uint32_t)q_blocks, q_geometry.grid.x, k_geometry.grid.x};
     const dim3 grid((uint32_t)(q_blocks + k_blocks));
     hipStream_t hip_stream = static_cast<hipStream_t>(stream);
