@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_reference_side_binding_lists_every_declared_function():
-    """The Rust `extern "C"` block a maintainer would add names every function of the header."""
+    """The Rust `extern "C"` block a maintainer would add, kept beside the header in the integration notes, names every function of the header."""
     header = open(os.path.join(ROOT, "include", "khm_gqa_sdpa.h")).read()
     header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
     declared = set(re.findall(r"\b(khm_[a-z0-9_]+)\s*\(", header))
