@@ -224,7 +224,7 @@ class Workload:
                                    page_table_index=fixed(0), num_active_tokens=fixed(shape.num_tokens),
                                    num_active_kv_splits=fixed(shape.num_sdpa_map_task_templates))
 
-            def launch_reduce():
+            def launch_reduce(gates=gates):
                 compute.invoke_reduce(partial_exp_sums=scratch.partial_exp_sums, partial_max_logits=scratch.partial_max_logits,
                                       partial_output=scratch.partial_output, cu_sdpa_partial_outputs=md.cu_sdpa_partial_outputs(),
                                       output=out, num_active_tokens=fixed(shape.num_tokens), gates=gates)
@@ -255,8 +255,8 @@ class Workload:
                 compute = sliced_q.Compute.new_direct(config, self.variant, qshape)
                 self._keep = (compute,)
 
-                def launch_map(pool):
-                    compute.invoke_direct(kv_pages=pool, output=out, **common)
+                def launch_map(pool, gates=gates):
+                    compute.invoke_direct(kv_pages=pool, output=out, gates=gates, **common)
 
                 launch_reduce = None
             else:
@@ -270,10 +270,10 @@ class Workload:
                     compute.invoke_map(kv_pages=pool, partial_output=partial, partial_exp_sums=sums, partial_max_logits=maxs,
                                        num_active_kv_splits=fixed(shape.num_sdpa_map_task_templates), **common)
 
-                def launch_reduce():
+                def launch_reduce(gates=gates):
                     compute.invoke_reduce(partial_output=partial, partial_exp_sums=sums, partial_max_logits=maxs,
                                           q_token_ranges=md.q_token_ranges(), cu_sdpa_partial_outputs=md.cu_sdpa_partial_outputs(),
-                                          output=out, num_active_q_token_tiles=fixed(shape.num_q_token_tiles))
+                                          output=out, num_active_q_token_tiles=fixed(shape.num_q_token_tiles), gates=gates)
 
                 if fused:
                     counters = torch.zeros(compute.arrival_counters_bytes(), dtype=torch.uint8, device=device)
@@ -586,6 +586,101 @@ def producer_rows(device, steps: int = 20) -> dict:
     return result
 
 
+def layer_rows(device, index: int, fp8_pages: bool = False, replays: int = 30) -> dict:
+    """Everything the reference's GQA::record enqueues between the input and the output projection
+    (crates/inference-executor-metal/src/attn/gqa/backend.rs:358-421) for one batch of a benchmark config, recorded twice
+    into a HIP graph and replayed: as the seven operators of the reference (projection split, Q norm + RoPE, K norm + RoPE,
+    K/V page write, Map, Reduce, gate; Map writes the output itself when the selector says so), and as the shortest recording
+    of this library (projection kernel, Map, gated Reduce or gated direct output).  Both leave the same bytes."""
+    import torch
+
+    from khalamari_amd import activation_gate, kv_page_write, projection_norm_rope_page_write, qgkv_split, rms_norm_rope
+    from khalamari_amd._lib import DTYPE_BF16, DTYPE_FP8_E4M3FN, ReplayU32
+
+    workload = Workload(index, device, num_pools=1, fp8_pages=fp8_pages)
+    spec = workload.spec
+    hq, hkv, d, tokens = spec["hq"], spec["hkv"], spec["d"], workload.num_tokens
+    if workload.fused:
+        raise RuntimeError("the layer recordings are timed on configs whose Map and Reduce are separate launches")
+    pool = workload.kv_pools[0]
+    generator = torch.Generator(device=device)
+    generator.manual_seed(78)
+    split_config = qgkv_split.Config.bf16(hq, hkv, d)
+    projection = torch.randn((tokens, split_config.projection_width()), device=device, dtype=torch.bfloat16, generator=generator)
+    rows = lambda heads: torch.empty((tokens, heads, d), device=device, dtype=torch.bfloat16)  # noqa: E731
+    q_split, g_rows, k_split, v_split, k_normed, gated_out = rows(hq), rows(hq), rows(hkv), rows(hkv), rows(hkv), rows(hq)
+    weight = torch.ones(d, device=device, dtype=torch.bfloat16)
+    positions = torch.tensor([h + i for h, n in zip(workload.histories, workload.q_lens) for i in range(n)], dtype=torch.int32, device=device)
+    req_slots = workload.metadata.req_slots()
+    blocks = workload.table_host.shape[1]
+    page_config = kv_page_write.Config(hkv, d, workload.page_bytes, kv_dtype=DTYPE_FP8_E4M3FN if fp8_pages else DTYPE_BF16)
+    page_shape = kv_page_write.Shape(tokens, kv_page_write.PageTableLayout(len(workload.histories), 1, blocks, 1))
+    q_config, k_config = rms_norm_rope.Config.bf16(hq, d, d, 1e-6, 1_000_000.0), rms_norm_rope.Config.bf16(hkv, d, d, 1e-6, 1_000_000.0)
+    split, q_norm, k_norm = qgkv_split.Compute(split_config), rms_norm_rope.Compute(q_config), rms_norm_rope.Compute(k_config)
+    writer = kv_page_write.Compute(page_config)
+    prologue = projection_norm_rope_page_write.Compute(q_config, k_config, page_config)
+    active, layer = ReplayU32.fixed(tokens), ReplayU32.fixed(0)
+
+    def seven_operators():
+        split.invoke(qgkv_split.Shape(tokens), qgkv=projection, q=q_split, g=g_rows, k=k_split, v=v_split, num_active_tokens=active)
+        q_norm.invoke(rms_norm_rope.Shape(tokens), input=q_split, norm_weight=weight, flat_token_indices=positions, output=workload.q,
+                      num_active_tokens=active)
+        k_norm.invoke(rms_norm_rope.Shape(tokens), input=k_split, norm_weight=weight, flat_token_indices=positions, output=k_normed,
+                      num_active_tokens=active)
+        writer.invoke(page_shape, pages=pool, flat_k=k_normed, flat_v=v_split, req_slots=req_slots, flat_token_indices=positions,
+                      page_ids=workload.page_table, num_active_token_writes=active, page_table_index=layer)
+        if workload.launch_reduce is None:
+            workload.launch_map(pool, gates=None)
+        else:
+            workload.launch_map(pool)
+            workload.launch_reduce(gates=None)
+        activation_gate.invoke(DTYPE_BF16, hq, d, tokens, workload.out, g_rows, gated_out, active)
+
+    def shortest():
+        prologue.invoke(page_shape, projection=projection, q_norm_weight=weight, k_norm_weight=weight, q_output=workload.q, gate_output=g_rows,
+                        pages=pool, req_slots=req_slots, flat_token_indices=positions, page_ids=workload.page_table, num_active_tokens=active,
+                        page_table_index=layer)
+        if workload.launch_reduce is None:
+            workload.launch_map(pool, gates=g_rows)
+        else:
+            workload.launch_map(pool)
+            workload.launch_reduce(gates=g_rows)
+
+    def replayed(record):
+        import gc
+
+        record()
+        torch.cuda.synchronize()
+        result = workload.out.clone() if record is shortest else gated_out.clone()
+        pages_after = pool.clone()
+        gc.collect()
+        graph = torch.cuda.CUDAGraph()
+        gc.disable()   # a collector run inside the capture could free device memory, which invalidates it
+        try:
+            with torch.cuda.graph(graph):
+                record()
+        finally:
+            gc.enable()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        begin.record()
+        for _ in range(replays):
+            graph.replay()
+        end.record()
+        torch.cuda.synchronize()
+        return begin.elapsed_time(end) * 1e3 / replays, result, pages_after
+
+    seven_us, seven_out, seven_pages = replayed(seven_operators)
+    short_us, short_out, short_pages = replayed(shortest)
+    return {"workload": spec["name"] + (" [FP8 E4M3FN pages]" if fp8_pages else ""), "tokens": tokens,
+            "launches_reference_recording": 7 if workload.launch_reduce is not None else 6,
+            "launches_shortest_recording": 3 if workload.launch_reduce is not None else 2,
+            "reference_recording_us": seven_us, "shortest_recording_us": short_us,
+            "same_output_bytes": bool(torch.equal(seven_out, short_out)), "same_page_bytes": bool(torch.equal(seven_pages, short_pages))}
+
+
 def slab_run_table(device, index: int = 2, steps: int = 40) -> list:
     """The read-only launch of a config's K/V bytes as contiguous runs of 4 .. 64 KB at random places of its pools: what a
     block that covered several KV heads of a page (longer contiguous reads) could gain over 4 KB slabs."""
@@ -653,6 +748,9 @@ def main() -> int:
                         help="time only the kernels that feed the SDPA (RMSNorm + RoPE, K/V page write) and print their JSON (profiling runs)")
     parser.add_argument("--fp8-pages", action="store_true",
                         help="headline config on FP8 E4M3FN pages, the reference's cache format (profiling runs; the default headline keeps bf16 pages)")
+    parser.add_argument("--layer", action="store_true",
+                        help="time the whole layer between the projections (producers, SDPA, gate) of --config N, as the reference's "
+                             "seven operators and as this library's shortest recording, replayed from a HIP graph")
     parser.add_argument("--slab-runs", action="store_true",
                         help="time only the read-only launch of the headline config's K/V bytes as contiguous runs of 4 .. 64 KB and print the table as JSON")
     parser.add_argument("--no-clock-probe", action="store_true", help="accepted and ignored (older command lines)")
@@ -676,6 +774,9 @@ def main() -> int:
         return 0
     if args.slab_runs:
         print(json.dumps({"slab_runs": slab_run_table(device, args.config)}))
+        return 0
+    if args.layer:
+        print(json.dumps({"layer": layer_rows(device, args.config, fp8_pages=args.fp8_pages)}))
         return 0
     headline = Workload(args.config, device, fp8_pages=args.fp8_pages)
     head = headline.report(args.steps, args.warmup)
