@@ -306,7 +306,7 @@ extern "C" int khm_bidi_block_sdpa(const khm_bidi_block_sdpa_config* config, con
     else if (chunks <= 2) kernel = f32 ? bidi_block_sdpa_kernel<float, 2> : bidi_block_sdpa_kernel<uint16_t, 2>;
     else if (chunks <= 4) kernel = f32 ? bidi_block_sdpa_kernel<float, 4> : bidi_block_sdpa_kernel<uint16_t, 4>;
     else kernel = f32 ? bidi_block_sdpa_kernel<float, 8> : bidi_block_sdpa_kernel<uint16_t, 8>;
-    hipLaunchKernelGGL(kernel, grid, dim3(kBidiThreads), lds_bytes, static_cast<hipStream_t>(stream), p, key_tile);
+    KHM_LAUNCH(kernel, grid, dim3(kBidiThreads), lds_bytes, static_cast<hipStream_t>(stream), p, key_tile);
     const hipError_t status = hipGetLastError();
     if (status != hipSuccess) return fail(KHM_ERR_HIP, "bidirectional block SDPA launch failed: %s", hipGetErrorString(status));
     return KHM_OK;

@@ -30,6 +30,16 @@ inline void clear_error() { last_error_storage().clear(); }
         if (!(condition)) return ::khm::fail(KHM_ERR_INVALID_ARGUMENT, __VA_ARGS__); \
     } while (0)
 
+// A kernel launch whose status the caller reads with hipGetLastError() afterwards.  The runtime keeps a thread's last error
+// until somebody reads it, whoever caused it (a failed copy or query of the host program's, say; without this, a launch
+// after such a call was reported as "launch failed: invalid argument"): it is read away first, so that the check after
+// the launch reports this launch and nothing older.  (Expands only in sources that include the HIP runtime header.)
+#define KHM_LAUNCH(...)                  \
+    do {                                 \
+        (void)hipGetLastError();         \
+        hipLaunchKernelGGL(__VA_ARGS__); \
+    } while (0)
+
 inline uint32_t div_ceil_u32(uint32_t a, uint32_t b) { return a / b + (a % b != 0); }
 inline uint64_t div_ceil_u64(uint64_t a, uint64_t b) { return a / b + (a % b != 0); }
 

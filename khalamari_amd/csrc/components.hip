@@ -131,10 +131,10 @@ static void launch_reduce_kernel(const khm_gqa_sdpa_config& config, const khm_gq
     if (few) {
         const uint64_t rows = (uint64_t)units * max_q_tokens * config.num_q_heads;
         const uint32_t rows_per_block = kReduceThreads / (config.head_dim / 4);
-        hipLaunchKernelGGL(select_reduce_rows_kernel(config.head_dim, ranged), dim3((uint32_t)((rows + rows_per_block - 1) / rows_per_block)),
+        KHM_LAUNCH(select_reduce_rows_kernel(config.head_dim, ranged), dim3((uint32_t)((rows + rows_per_block - 1) / rows_per_block)),
                            dim3(kReduceThreads), 0, stream, p);
     } else {
-        hipLaunchKernelGGL(sliced, dim3(units * max_q_tokens, config.num_q_heads, 1), dim3(kReduceThreads), 0, stream, p);
+        KHM_LAUNCH(sliced, dim3(units * max_q_tokens, config.num_q_heads, 1), dim3(kReduceThreads), 0, stream, p);
     }
 }
 
@@ -391,7 +391,7 @@ static int launch_sliced_kv_map(const khm_sliced_kv* compute, const khm_sliced_k
         p.gates = fused->gates;
     }
     const dim3 grid(shape.num_total_sdpa_map_task_templates, config.num_kv_heads * compute->num_q_head_ranges, 1);
-    hipLaunchKernelGGL(compute->map, grid, dim3(kMapWaves * 64), 0, static_cast<hipStream_t>(stream), p);
+    KHM_LAUNCH(compute->map, grid, dim3(kMapWaves * 64), 0, static_cast<hipStream_t>(stream), p);
     return check_launch("sliced-KV map");
 }
 
@@ -506,7 +506,7 @@ extern "C" int khm_sliced_kv_map_reduce_static(const khm_sliced_kv* compute, con
     // GPU and an earlier call may have been abandoned half-way, so they are cleared here - by a kernel, not a memset
     // node, so that the call can be captured into a HIP graph.
     const uint32_t counters = (uint32_t)(counter_bytes / 4);
-    hipLaunchKernelGGL(clear_u32_kernel, dim3((counters + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream),
+    KHM_LAUNCH(clear_u32_kernel, dim3((counters + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream),
                        reinterpret_cast<uint32_t*>(base), counters);
     if (int s = check_launch("static scratch clear")) return s;
     const FusedReduceArgs fused{static_cast<const uint32_t*>(buffers->cu_sdpa_partial_outputs.ptr), reinterpret_cast<uint32_t*>(base),
@@ -683,7 +683,7 @@ static int launch_sliced_q_map(const khm_sliced_q* compute, const khm_buffer& q,
         p.gates = fused->gates;
     }
     const dim3 grid(shape.num_total_sdpa_map_task_templates, config.num_kv_heads * compute->num_q_head_ranges, 1);
-    hipLaunchKernelGGL(compute->map, grid, dim3(compute->map_threads), compute->map_smem_bytes, static_cast<hipStream_t>(stream), p);
+    KHM_LAUNCH(compute->map, grid, dim3(compute->map_threads), compute->map_smem_bytes, static_cast<hipStream_t>(stream), p);
     return check_launch("sliced-Q map");
 }
 
@@ -845,11 +845,11 @@ extern "C" int khm_gqa_activation_gate(uint32_t dtype, uint32_t num_q_heads, uin
     if (address_bits % 16 == 0) {
         const uint64_t per_block = 256ull * gate_elements_per_thread(p.is_f32 != 0);
         const uint32_t blocks = (uint32_t)((values + per_block - 1) / per_block);
-        if (p.is_f32) hipLaunchKernelGGL(activation_gate_vector_kernel<true>, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), p);
-        else hipLaunchKernelGGL(activation_gate_vector_kernel<false>, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+        if (p.is_f32) KHM_LAUNCH(activation_gate_vector_kernel<true>, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+        else KHM_LAUNCH(activation_gate_vector_kernel<false>, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), p);
         return check_launch("activation gate");
     }
     const uint32_t blocks = (uint32_t)((values + 255) / 256);
-    hipLaunchKernelGGL(activation_gate_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    KHM_LAUNCH(activation_gate_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), p);
     return check_launch("activation gate");
 }

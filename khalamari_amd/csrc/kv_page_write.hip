@@ -224,9 +224,9 @@ extern "C" int khm_kv_page_write(const khm_kv_page_write_config* config, const k
     KHM_REQUIRE(chunk_blocks <= 65535, "GQA KV page write: %llu chunks per token write exceed the launch grid", (unsigned long long)chunks_per_write);
     const dim3 grid((shape->num_total_token_writes + kWritesPerBlock - 1) / kWritesPerBlock, (uint32_t)chunk_blocks);
     if (config->kv_dtype == KHM_DTYPE_FP8_E4M3FN) {
-        hipLaunchKernelGGL(kv_page_write_kernel<true>, grid, dim3(block_threads), 0, static_cast<hipStream_t>(stream), p);
+        KHM_LAUNCH(kv_page_write_kernel<true>, grid, dim3(block_threads), 0, static_cast<hipStream_t>(stream), p);
     } else {
-        hipLaunchKernelGGL(kv_page_write_kernel<false>, grid, dim3(block_threads), 0, static_cast<hipStream_t>(stream), p);
+        KHM_LAUNCH(kv_page_write_kernel<false>, grid, dim3(block_threads), 0, static_cast<hipStream_t>(stream), p);
     }
     return check_page_write_launch("KV page write");
 }
@@ -241,7 +241,7 @@ extern "C" int khm_fp8_e4m3_to_bf16_device(khm_buffer codes, khm_buffer bf16_out
     KHM_REQUIRE(reinterpret_cast<uintptr_t>(codes.ptr) % 8 == 0 && reinterpret_cast<uintptr_t>(bf16_out.ptr) % 16 == 0,
                 "FP8 decode buffers must be 8- and 16-byte aligned");
     const uint64_t threads = (count + 7) / 8;
-    hipLaunchKernelGGL(fp8_decode_kernel, dim3((uint32_t)((threads + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+    KHM_LAUNCH(fp8_decode_kernel, dim3((uint32_t)((threads + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint8_t*>(codes.ptr), static_cast<uint16_t*>(bf16_out.ptr), count);
     return check_page_write_launch("FP8 decode");
 }
@@ -256,7 +256,7 @@ extern "C" int khm_bf16_to_fp8_e4m3_device(khm_buffer bf16_in, khm_buffer codes,
     KHM_REQUIRE(reinterpret_cast<uintptr_t>(codes.ptr) % 8 == 0 && reinterpret_cast<uintptr_t>(bf16_in.ptr) % 16 == 0,
                 "FP8 encode buffers must be 8- and 16-byte aligned");
     const uint64_t threads = (count + 7) / 8;
-    hipLaunchKernelGGL(fp8_encode_kernel, dim3((uint32_t)((threads + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+    KHM_LAUNCH(fp8_encode_kernel, dim3((uint32_t)((threads + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint16_t*>(bf16_in.ptr), static_cast<uint8_t*>(codes.ptr), count);
     return check_page_write_launch("FP8 encode");
 }

@@ -110,10 +110,10 @@ static uint32_t unit_bytes_for(uint64_t head_row_bytes, const khm_buffer* const*
 template <bool GATED>
 static void launch_split(uint32_t unit_bytes, dim3 grid, hipStream_t stream, const SplitParams& p) {
     switch (unit_bytes) {
-        case 16: hipLaunchKernelGGL((projection_split_kernel<uint4, GATED>), grid, dim3(256), 0, stream, p); break;
-        case 8: hipLaunchKernelGGL((projection_split_kernel<uint2, GATED>), grid, dim3(256), 0, stream, p); break;
-        case 4: hipLaunchKernelGGL((projection_split_kernel<uint32_t, GATED>), grid, dim3(256), 0, stream, p); break;
-        default: hipLaunchKernelGGL((projection_split_kernel<uint16_t, GATED>), grid, dim3(256), 0, stream, p); break;
+        case 16: KHM_LAUNCH((projection_split_kernel<uint4, GATED>), grid, dim3(256), 0, stream, p); break;
+        case 8: KHM_LAUNCH((projection_split_kernel<uint2, GATED>), grid, dim3(256), 0, stream, p); break;
+        case 4: KHM_LAUNCH((projection_split_kernel<uint32_t, GATED>), grid, dim3(256), 0, stream, p); break;
+        default: KHM_LAUNCH((projection_split_kernel<uint16_t, GATED>), grid, dim3(256), 0, stream, p); break;
     }
 }
 

@@ -582,7 +582,7 @@ extern "C" int khm_rms_norm_rope(const khm_rms_norm_rope_config* config, uint32_
             typedef decltype(weight_tag) W;
 #define KHM_ROWS_CASE(LPR, PARTNER)                                                                                        \
     if (geometry.lanes_per_row == LPR && geometry.partner == PARTNER) {                                                    \
-        hipLaunchKernelGGL((rms_norm_rope_rows_kernel<T, W, LPR, PARTNER>), geometry.grid, dim3(256), 0, hip_stream, p);    \
+        KHM_LAUNCH((rms_norm_rope_rows_kernel<T, W, LPR, PARTNER>), geometry.grid, dim3(256), 0, hip_stream, p);    \
         return;                                                                                                            \
     }
             KHM_ROWS_CASES(KHM_ROWS_CASE)
@@ -594,10 +594,10 @@ extern "C" int khm_rms_norm_rope(const khm_rms_norm_rope_config* config, uint32_
         else launch(float{}, float{});
     } else {
         const dim3 grid(num_total_tokens * config->num_heads);
-        if (io_bf16 && weight_bf16) hipLaunchKernelGGL((rms_norm_rope_kernel<uint16_t, uint16_t>), grid, dim3(64), 0, hip_stream, p);
-        else if (io_bf16) hipLaunchKernelGGL((rms_norm_rope_kernel<uint16_t, float>), grid, dim3(64), 0, hip_stream, p);
-        else if (weight_bf16) hipLaunchKernelGGL((rms_norm_rope_kernel<float, uint16_t>), grid, dim3(64), 0, hip_stream, p);
-        else hipLaunchKernelGGL((rms_norm_rope_kernel<float, float>), grid, dim3(64), 0, hip_stream, p);
+        if (io_bf16 && weight_bf16) KHM_LAUNCH((rms_norm_rope_kernel<uint16_t, uint16_t>), grid, dim3(64), 0, hip_stream, p);
+        else if (io_bf16) KHM_LAUNCH((rms_norm_rope_kernel<uint16_t, float>), grid, dim3(64), 0, hip_stream, p);
+        else if (weight_bf16) KHM_LAUNCH((rms_norm_rope_kernel<float, uint16_t>), grid, dim3(64), 0, hip_stream, p);
+        else KHM_LAUNCH((rms_norm_rope_kernel<float, float>), grid, dim3(64), 0, hip_stream, p);
     }
     const hipError_t status = hipGetLastError();
     if (status != hipSuccess) return fail(KHM_ERR_HIP, "RMSNorm/RoPE launch failed: %s", hipGetErrorString(status));
@@ -641,7 +641,7 @@ extern "C" int khm_k_norm_rope_page_write(const khm_rms_norm_rope_config* norm_c
         constexpr bool FP8 = decltype(fp8_tag)::value;
 #define KHM_ROWS_CASE(LPR, PARTNER)                                                                                                    \
     if (geometry.lanes_per_row == LPR && geometry.partner == PARTNER) {                                                                \
-        hipLaunchKernelGGL((k_norm_rope_page_write_kernel<W, LPR, PARTNER, FP8>), geometry.grid, dim3(256), 0, hip_stream, p, pages);   \
+        KHM_LAUNCH((k_norm_rope_page_write_kernel<W, LPR, PARTNER, FP8>), geometry.grid, dim3(256), 0, hip_stream, p, pages);   \
         return;                                                                                                                        \
     }
         KHM_ROWS_CASES(KHM_ROWS_CASE)
@@ -745,7 +745,7 @@ extern "C" int khm_gqa_projection_norm_rope_page_write(uint32_t gated, const khm
         constexpr bool FP8 = decltype(fp8_tag)::value, GATED = decltype(gated_tag)::value;
 #define KHM_ROWS_CASE(LPR, PARTNER)                                                                                                          \
     if (q_geometry.lanes_per_row == LPR && q_geometry.partner == PARTNER) {                                                                  \
-        hipLaunchKernelGGL((projection_norm_rope_page_write_kernel<W, LPR, PARTNER, FP8, GATED>), grid, dim3(256), 0, hip_stream, p, k_role, \
+        KHM_LAUNCH((projection_norm_rope_page_write_kernel<W, LPR, PARTNER, FP8, GATED>), grid, dim3(256), 0, hip_stream, p, k_role, \
                            pages, blocks);                                                                                                   \
         return;                                                                                                                              \
     }
